@@ -1,0 +1,153 @@
+/*
+ * sfno_spectral.h -- C ABI of the MI355X (gfx950) SFNO spectral hot path.
+ *
+ * The library replaces, for one GPU, the device work that Makani's SFNO issues
+ * through torch-harmonics and torch.einsum:
+ *   - RealSHT.forward / InverseRealSHT.forward (torch-harmonics; constructed at
+ *     makani/models/networks/sfnonet.py:536-539, called at
+ *     makani/models/common/spectral_convolution.py:131,133,141 and
+ *     makani/models/networks/sfnonet.py:596,598,616),
+ *   - the "dhconv" contraction, makani/models/common/contractions.py:130-136
+ *     (selected by makani/models/common/factorizations.py:212-232).
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative SFNO_E* code; nothing throws.
+ *   - all device pointers are plain HIP device addresses owned by the caller;
+ *     `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *   - the compute entry points only enqueue kernels on `stream`: they do not
+ *     allocate, free, synchronise or create streams.  Scratch memory is passed in by
+ *     the caller (`workspace`), sized by the matching *_workspace_bytes query.
+ *   - "rows" is the product of all leading dimensions (batch x channels).
+ *   - real fields are float32 [rows][nlat][nlon]; coefficients are complex64
+ *     (interleaved re,im) [rows][lmax][mmax], m fastest -- the memory layout the
+ *     reference modules produce.
+ *   - the "spectral" layout is the library's internal, order-major coefficient
+ *     layout float32 [mmax][lmax][ld] with ld = sfno_spectral_ld(rows) and the
+ *     channel axis holding (re,im) of row r at 2r, 2r+1.  Entries with l < m are
+ *     never read and never written.
+ */
+#ifndef SFNO_SPECTRAL_H
+#define SFNO_SPECTRAL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* error codes */
+#define SFNO_OK 0
+#define SFNO_EINVAL (-1)    /* bad argument (shape, enum, null pointer) */
+#define SFNO_ENOMEM (-2)    /* device or host allocation failed at plan creation */
+#define SFNO_EHIP (-3)      /* a HIP runtime call failed */
+#define SFNO_EWORKSPACE (-4) /* workspace too small */
+#define SFNO_EUNSUPPORTED (-5)
+
+/* grid = quadrature rule in latitude (torch-harmonics `grid=` strings) */
+#define SFNO_GRID_LEGENDRE_GAUSS 0
+#define SFNO_GRID_LOBATTO 1
+#define SFNO_GRID_EQUIANGULAR 2
+
+/* norm = normalisation of the harmonics (torch-harmonics `norm=` strings) */
+#define SFNO_NORM_ORTHO 0
+#define SFNO_NORM_FOUR_PI 1
+#define SFNO_NORM_SCHMIDT 2
+
+/* which tables a plan holds */
+#define SFNO_DIR_FORWARD 1
+#define SFNO_DIR_INVERSE 2
+
+/* arithmetic of the Legendre / channel-mix contractions */
+#define SFNO_COMPUTE_FP32 0      /* fp32 MFMA, fp32 tables */
+#define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs, fp32 accumulate */
+
+typedef struct sfno_sht_plan sfno_sht_plan;
+typedef struct sfno_dhconv_weights sfno_dhconv_weights;
+
+const char* sfno_strerror(int code);
+/* library ABI version, bumped on any signature change */
+int sfno_version(void);
+
+/* ---- host-only helpers (no GPU needed) ------------------------------------------- */
+
+/* Colatitudes theta[nlat] (ascending: row 0 is the northernmost) and quadrature
+ * weights w[nlat] of a grid.  Replaces torch_harmonics.quadrature.{legendre_gauss,
+ * lobatto,clenshaw_curtiss}_weights as called by the transform constructors and by
+ * makani/utils/grids.py:32,77,83. */
+int sfno_quadrature(int grid, int nlat, double* theta, double* w);
+
+/* Dense float64 table out[m][l][k] = Pbar_l^m(cos theta[k]) (zero for l < m), the
+ * tensor the reference modules keep as the buffers `weights` (after multiplication by
+ * w[k]) and `pct`.  `inverse` selects the synthesis normalisation. */
+int sfno_legendre_table(int mmax, int lmax, int nlat, const double* theta, int norm,
+                        int inverse, int csphase, double* out);
+
+/* ---- transform plans --------------------------------------------------------------- */
+
+/* Builds the packed Legendre tables and FFT twiddles on the current HIP device.
+ * Mirrors RealSHT.__init__ / InverseRealSHT.__init__(nlat, nlon, lmax, mmax, grid, norm,
+ * csphase); `directions` is a mask of SFNO_DIR_*; `compute` one of SFNO_COMPUTE_*. */
+int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int grid, int norm,
+                         int csphase, int directions, int compute, sfno_sht_plan** out);
+int sfno_sht_plan_destroy(sfno_sht_plan* plan);
+
+/* leading dimension (floats) of the channel axis of the spectral layout */
+int64_t sfno_spectral_ld(int64_t rows);
+/* floats in one spectral-layout buffer: mmax * lmax * ld */
+int64_t sfno_spectral_elems(const sfno_sht_plan* plan, int64_t rows);
+
+/* bytes of scratch the calls below need for `rows` rows */
+size_t sfno_sht_workspace_bytes(const sfno_sht_plan* plan, int64_t rows);
+
+/* RealSHT.forward: x float32 [rows][nlat][nlon] -> coeffs complex64 [rows][lmax][mmax] */
+int sfno_sht_forward(const sfno_sht_plan* plan, const float* x, void* coeffs, int64_t rows,
+                     void* workspace, size_t workspace_bytes, void* stream);
+/* InverseRealSHT.forward: coeffs complex64 [rows][lmax][mmax] -> x float32 [rows][nlat][nlon] */
+int sfno_sht_inverse(const sfno_sht_plan* plan, const void* coeffs, float* x, int64_t rows,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same transforms with coefficients kept in the spectral layout (no layout pass). */
+int sfno_sht_analysis(const sfno_sht_plan* plan, const float* x, float* spec, int64_t rows,
+                      void* workspace, size_t workspace_bytes, void* stream);
+int sfno_sht_synthesis(const sfno_sht_plan* plan, const float* spec, float* x, int64_t rows,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* layout passes between the reference coefficient layout and the spectral layout */
+/* `triangular` != 0: only entries with m <= l are moved (to_coeffs writes zeros for
+ * m > l); 0: the whole lmax x mmax rectangle is moved. */
+int sfno_coeffs_to_spectral(const void* coeffs, float* spec, int64_t rows, int lmax, int mmax,
+                            int triangular, void* stream);
+int sfno_spectral_to_coeffs(const float* spec, void* coeffs, int64_t rows, int lmax, int mmax,
+                            int triangular, void* stream);
+
+/* ---- dhconv ------------------------------------------------------------------------ */
+
+/* Packs a SpectralConv weight (complex64 [I][O][L], l fastest: the parameter layout of
+ * makani/models/common/spectral_convolution.py:73-102) into the per-degree MFMA operand
+ * stream.  Allocates device memory owned by the handle. */
+int sfno_dhconv_weights_create(int in_channels, int out_channels, int lmax, int compute,
+                               sfno_dhconv_weights** out);
+/* (re)fill the packed stream from the current value of the parameter; enqueue only */
+int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream);
+int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w);
+
+/* y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l] on spectral-layout buffers:
+ * spec_in rows = batch*in_channels, spec_out rows = batch*out_channels.  With
+ * `triangular` != 0 only m <= l is read and written (coefficients of a forward
+ * transform are zero elsewhere).  Replaces _contract_dhconv (contractions.py:130-136). */
+int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* spec_in, float* spec_out,
+                         int batch, int mmax, int triangular, void* stream);
+
+/* Same contraction on the reference layout: x complex64 [B][I][L][M] -> y complex64
+ * [B][O][L][M] (contiguous), as the callable returned by get_contract_fun
+ * (factorizations.py:229-232) computes it.  `triangular` as above (then y is zero for
+ * m > l, which equals the reference result whenever x is zero there). */
+size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int mmax);
+int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y, int batch, int mmax,
+                int triangular, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SFNO_SPECTRAL_H */

@@ -1,0 +1,306 @@
+// C ABI of libsfno_spectral: plan management and the enqueue-only compute entry points.
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "sfno_internal.h"
+
+using namespace sfno;
+
+namespace {
+
+const int kVersion = 1;
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+template <class T>
+int upload(T** dst, const std::vector<T>& src) {
+    *dst = nullptr;
+    size_t bytes = sizeof(T) * std::max<size_t>(src.size(), 1);
+    if (hipMalloc((void**)dst, bytes) != hipSuccess) return SFNO_ENOMEM;
+    if (!src.empty() && hipMemcpy(*dst, src.data(), sizeof(T) * src.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
+    return SFNO_OK;
+}
+
+void free_table(PgemmTable& t) {
+    if (t.d_A) (void)hipFree(t.d_A);
+    if (t.d_aoff) (void)hipFree(t.d_aoff);
+    if (t.d_work) (void)hipFree(t.d_work);
+    t = PgemmTable();
+}
+
+int build_legendre_table(const sfno_sht_plan& p, const double* theta, const double* quad_w, bool analysis, PgemmTable& t) {
+    LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, analysis ? 0 : 1, p.csphase);
+    std::vector<float> packed;
+    std::vector<int64_t> aoff;
+    pack_legendre(gen, quad_w, analysis, packed, aoff);
+    std::vector<int> nrb(p.mmax);
+    std::vector<double> cost(p.mmax);
+    for (int m = 0; m < p.mmax; ++m) {
+        int nl = std::max(0, p.lmax - m);
+        if (analysis) {
+            nrb[m] = (nl + PG_ROWS - 1) / PG_ROWS;
+            cost[m] = 1.0;
+        } else {
+            nrb[m] = (p.nlat + PG_ROWS - 1) / PG_ROWS;    // orders without any degree still zero-fill their rows
+            cost[m] = 1.0 + (nl + PG_KC - 1) / PG_KC;
+        }
+    }
+    std::vector<int2> work;
+    build_worklist(nrb, cost, work);
+    t.n_work = (int)work.size();
+    t.n_blocks = (int64_t)(packed.size() / PG_BLOCK_FLOATS);
+    int rc;
+    if ((rc = upload(&t.d_A, packed)) != SFNO_OK) return rc;
+    if ((rc = upload(&t.d_aoff, aoff)) != SFNO_OK) return rc;
+    if ((rc = upload(&t.d_work, work)) != SFNO_OK) return rc;
+    return SFNO_OK;
+}
+
+struct Ws {
+    float* xm;
+    float* spec;
+    size_t bytes;
+};
+
+Ws carve(const sfno_sht_plan* p, int64_t rows, void* base) {
+    const int64_t ld = sfno_spectral_ld(rows);
+    Ws w;
+    size_t xm_bytes = align_up(sizeof(float) * (size_t)p->mmax * p->nlat * ld, 256);
+    size_t spec_bytes = align_up(sizeof(float) * (size_t)p->mmax * p->lmax * ld, 256);
+    w.xm = reinterpret_cast<float*>(base);
+    w.spec = reinterpret_cast<float*>(reinterpret_cast<char*>(base) + xm_bytes);
+    w.bytes = xm_bytes + spec_bytes;
+    return w;
+}
+
+PgemmArgs legendre_args(const sfno_sht_plan* p, const PgemmTable& t, const float* q, float* out, int64_t ld) {
+    PgemmArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.A = t.d_A;
+    a.a_off = t.d_aoff;
+    a.work = t.d_work;
+    a.Q = q;
+    a.Out = out;
+    a.lmax = p->lmax;
+    a.nlat = p->nlat;
+    a.mmax = p->mmax;
+    a.ld = (int)ld;
+    return a;
+}
+
+bool rows_ok(int64_t rows) { return rows > 0 && sfno_spectral_ld(rows) < (int64_t)1 << 30; }
+
+}  // namespace
+
+extern "C" const char* sfno_strerror(int code) {
+    switch (code) {
+        case SFNO_OK: return "ok";
+        case SFNO_EINVAL: return "invalid argument";
+        case SFNO_ENOMEM: return "out of memory";
+        case SFNO_EHIP: return "HIP runtime error";
+        case SFNO_EWORKSPACE: return "workspace too small";
+        case SFNO_EUNSUPPORTED: return "unsupported configuration";
+    }
+    return "unknown error";
+}
+
+extern "C" int sfno_version(void) { return kVersion; }
+
+extern "C" int64_t sfno_spectral_ld(int64_t rows) { return (2 * rows + 3) / 4 * 4; }
+
+extern "C" int64_t sfno_spectral_elems(const sfno_sht_plan* p, int64_t rows) {
+    if (!p || rows <= 0) return 0;
+    return (int64_t)p->mmax * p->lmax * sfno_spectral_ld(rows);
+}
+
+extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int grid, int norm, int csphase, int directions,
+                                    int compute, sfno_sht_plan** out) {
+    if (!out) return SFNO_EINVAL;
+    *out = nullptr;
+    if (nlat < 2 || nlon < 1 || lmax < 1 || mmax < 1) return SFNO_EINVAL;
+    if (mmax > nlon / 2 + 1) return SFNO_EINVAL;
+    if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
+    if (!(directions & (SFNO_DIR_FORWARD | SFNO_DIR_INVERSE))) return SFNO_EINVAL;
+    if (compute != SFNO_COMPUTE_FP32) return SFNO_EUNSUPPORTED;
+    sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
+    if (!p) return SFNO_ENOMEM;
+    p->nlat = nlat; p->nlon = nlon; p->lmax = lmax; p->mmax = mmax;
+    p->grid = grid; p->norm = norm; p->csphase = csphase ? 1 : 0;
+    p->directions = directions; p->compute = compute;
+    if (hipGetDevice(&p->device) != hipSuccess) { delete p; return SFNO_EHIP; }
+    std::vector<double> theta(nlat), w(nlat);
+    int rc = quadrature(grid, nlat, theta.data(), w.data());
+    if (rc == SFNO_OK) rc = fft_plan_init(p->fft, nlon);
+    if (rc == SFNO_OK && (directions & SFNO_DIR_FORWARD)) rc = build_legendre_table(*p, theta.data(), w.data(), true, p->fwd);
+    if (rc == SFNO_OK && (directions & SFNO_DIR_INVERSE)) rc = build_legendre_table(*p, theta.data(), w.data(), false, p->inv);
+    if (rc != SFNO_OK) { sfno_sht_plan_destroy(p); return rc; }
+    *out = p;
+    return SFNO_OK;
+}
+
+extern "C" int sfno_sht_plan_destroy(sfno_sht_plan* p) {
+    if (!p) return SFNO_OK;
+    free_table(p->fwd);
+    free_table(p->inv);
+    fft_plan_free(p->fft);
+    delete p;
+    return SFNO_OK;
+}
+
+extern "C" size_t sfno_sht_workspace_bytes(const sfno_sht_plan* p, int64_t rows) {
+    if (!p || !rows_ok(rows)) return 0;
+    return carve(p, rows, nullptr).bytes;
+}
+
+extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const float* x, float* spec, int64_t rows, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+    if (!p || !x || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t ld = sfno_spectral_ld(rows);
+    int rc = rfft_launch(p->fft, x, w.xm, rows, p->nlat, p->mmax, (int)ld, s);
+    if (rc != SFNO_OK) return rc;
+    PgemmArgs a = legendre_args(p, p->fwd, w.xm, spec, ld);
+    return pgemm_launch(PG_ANALYSIS, a, p->fwd.n_work, ld, s);
+}
+
+extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, float* x, int64_t rows, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+    if (!p || !x || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t ld = sfno_spectral_ld(rows);
+    PgemmArgs a = legendre_args(p, p->inv, spec, w.xm, ld);
+    int rc = pgemm_launch(PG_SYNTHESIS, a, p->inv.n_work, ld, s);
+    if (rc != SFNO_OK) return rc;
+    return irfft_launch(p->fft, w.xm, x, rows, p->nlat, p->mmax, (int)ld, s);
+}
+
+extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* coeffs, int64_t rows, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!p || !coeffs || !rows_ok(rows)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = sfno_sht_analysis(p, x, w.spec, rows, workspace, workspace_bytes, stream);
+    if (rc != SFNO_OK) return rc;
+    return spectral_to_coeffs_launch(w.spec, reinterpret_cast<float2*>(coeffs), rows, p->lmax, p->mmax,
+                                     (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+}
+
+extern "C" int sfno_sht_inverse(const sfno_sht_plan* p, const void* coeffs, float* x, int64_t rows, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!p || !coeffs || !rows_ok(rows)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = coeffs_to_spectral_launch(reinterpret_cast<const float2*>(coeffs), w.spec, rows, p->lmax, p->mmax,
+                                       (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+    if (rc != SFNO_OK) return rc;
+    return sfno_sht_synthesis(p, w.spec, x, rows, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sfno_coeffs_to_spectral(const void* coeffs, float* spec, int64_t rows, int lmax, int mmax, int triangular,
+                                       void* stream) {
+    if (!coeffs || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    return coeffs_to_spectral_launch(reinterpret_cast<const float2*>(coeffs), spec, rows, lmax, mmax, (int)sfno_spectral_ld(rows),
+                                     triangular, (hipStream_t)stream);
+}
+
+extern "C" int sfno_spectral_to_coeffs(const float* spec, void* coeffs, int64_t rows, int lmax, int mmax, int triangular,
+                                       void* stream) {
+    if (!coeffs || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    return spectral_to_coeffs_launch(spec, reinterpret_cast<float2*>(coeffs), rows, lmax, mmax, (int)sfno_spectral_ld(rows),
+                                     triangular, (hipStream_t)stream);
+}
+
+// ---- dhconv -------------------------------------------------------------------------------------
+
+extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno_dhconv_weights** out) {
+    if (!out) return SFNO_EINVAL;
+    *out = nullptr;
+    if (I < 1 || O < 1 || L < 1) return SFNO_EINVAL;
+    if (compute != SFNO_COMPUTE_FP32) return SFNO_EUNSUPPORTED;
+    sfno_dhconv_weights* w = new (std::nothrow) sfno_dhconv_weights();
+    if (!w) return SFNO_ENOMEM;
+    w->I = I; w->O = O; w->L = L; w->compute = compute;
+    if (hipGetDevice(&w->device) != hipSuccess) { delete w; return SFNO_EHIP; }
+    w->nrb = (2 * O + PG_ROWS - 1) / PG_ROWS;
+    w->nc = (2 * I + PG_KC - 1) / PG_KC;
+    const int64_t per_l = (int64_t)w->nrb * w->nc;
+    w->tab.n_blocks = per_l * L;
+    std::vector<int64_t> aoff(L);
+    std::vector<int> nrb(L, w->nrb);
+    std::vector<double> cost(L);
+    for (int l = 0; l < L; ++l) {
+        aoff[l] = per_l * l;
+        cost[l] = 1.0 + l;      // a forward transform fills orders m <= l only
+    }
+    std::vector<int2> work;
+    build_worklist(nrb, cost, work);
+    w->tab.n_work = (int)work.size();
+    int rc = SFNO_OK;
+    if (hipMalloc((void**)&w->tab.d_A, sizeof(float) * (size_t)w->tab.n_blocks * PG_BLOCK_FLOATS) != hipSuccess) rc = SFNO_ENOMEM;
+    if (rc == SFNO_OK) rc = upload(&w->tab.d_aoff, aoff);
+    if (rc == SFNO_OK) rc = upload(&w->tab.d_work, work);
+    if (rc != SFNO_OK) { sfno_dhconv_weights_destroy(w); return rc; }
+    *out = w;
+    return SFNO_OK;
+}
+
+extern "C" int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream) {
+    if (!w || !weight) return SFNO_EINVAL;
+    return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->tab.d_A, w->I, w->O, w->L, (hipStream_t)stream);
+}
+
+extern "C" int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w) {
+    if (!w) return SFNO_OK;
+    free_table(w->tab);
+    delete w;
+    return SFNO_OK;
+}
+
+extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* spec_in, float* spec_out, int batch, int mmax,
+                                    int triangular, void* stream) {
+    if (!w || !spec_in || !spec_out || batch < 1 || mmax < 1) return SFNO_EINVAL;
+    PgemmArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.A = w->tab.d_A;
+    a.a_off = w->tab.d_aoff;
+    a.work = w->tab.d_work;
+    a.Q = spec_in;
+    a.Out = spec_out;
+    a.B = batch;
+    a.I2 = 2 * w->I;
+    a.O2 = 2 * w->O;
+    a.L = w->L;
+    a.M = mmax;
+    a.tri = triangular ? 1 : 0;
+    a.ld_in = (int)sfno_spectral_ld((int64_t)batch * w->I);
+    a.ld_out = (int)sfno_spectral_ld((int64_t)batch * w->O);
+    return pgemm_launch(PG_DHCONV, a, w->tab.n_work, (int64_t)mmax * batch, (hipStream_t)stream);
+}
+
+extern "C" size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int mmax) {
+    if (!w || batch < 1 || mmax < 1) return 0;
+    size_t in_b = align_up(sizeof(float) * (size_t)mmax * w->L * sfno_spectral_ld((int64_t)batch * w->I), 256);
+    size_t out_b = align_up(sizeof(float) * (size_t)mmax * w->L * sfno_spectral_ld((int64_t)batch * w->O), 256);
+    return in_b + out_b;
+}
+
+extern "C" int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y, int batch, int mmax, int triangular,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (!w || !x || !y || batch < 1 || mmax < 1) return SFNO_EINVAL;
+    if (!workspace || workspace_bytes < sfno_dhconv_workspace_bytes(w, batch, mmax)) return SFNO_EWORKSPACE;
+    size_t in_b = align_up(sizeof(float) * (size_t)mmax * w->L * sfno_spectral_ld((int64_t)batch * w->I), 256);
+    float* sin = reinterpret_cast<float*>(workspace);
+    float* sout = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + in_b);
+    int rc = sfno_coeffs_to_spectral(x, sin, (int64_t)batch * w->I, w->L, mmax, triangular, stream);
+    if (rc != SFNO_OK) return rc;
+    rc = sfno_dhconv_spectral(w, sin, sout, batch, mmax, triangular, stream);
+    if (rc != SFNO_OK) return rc;
+    return sfno_spectral_to_coeffs(sout, y, (int64_t)batch * w->O, w->L, mmax, triangular, stream);
+}

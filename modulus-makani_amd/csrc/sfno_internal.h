@@ -1,0 +1,97 @@
+// Internal declarations shared by the host code and the HIP kernels of libsfno_spectral.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <vector>
+
+#include "sfno_spectral.h"
+
+namespace sfno {
+
+// ---- packed-operand GEMM ("pgemm") ---------------------------------------------------
+// One operand of every contraction on this path is constant between calls (Legendre
+// table, SpectralConv weight).  It is stored as a stream of 32x16 blocks, each laid out
+// exactly as the MFMA fragments of one wavefront consume it: block = 2 halves x 64 lanes
+// x float4; lane j of half h holds, for s = 0..3,
+//     P[row = 32*rb + (j & 31)][k = 16*c + 8*h + 2*s + (j >> 5)].
+// A wavefront owns one 32-row block `rb` of one batch (order m or degree l) and walks its
+// K-chunks c = 0..nc-1, which are contiguous in memory.
+constexpr int PG_ROWS = 32;        // rows per block (MFMA 32x32x2)
+constexpr int PG_KC = 16;          // K per block
+constexpr int PG_BLOCK_FLOATS = PG_ROWS * PG_KC;   // 512 floats = 2 KiB
+constexpr int PG_WAVES = 4;        // wavefronts (= row blocks) per workgroup
+
+enum PgemmMode { PG_ANALYSIS = 0, PG_SYNTHESIS = 1, PG_DHCONV = 2 };
+
+struct PgemmTable {
+    float* d_A = nullptr;          // packed stream
+    int64_t* d_aoff = nullptr;     // [nbatch] first block of each batch
+    int2* d_work = nullptr;        // [n_work] {batch, first row block} per workgroup, -1 = idle
+    int n_work = 0;                // multiple of 8 (one queue per XCD, interleaved)
+    int64_t n_blocks = 0;
+};
+
+struct PgemmArgs {
+    const float* A;
+    const int64_t* a_off;
+    const int2* work;
+    const float* Q;
+    float* Out;
+    int lmax, nlat, mmax;          // Legendre modes
+    int ld;                        // channel leading dimension of Q and Out (Legendre modes)
+    // dhconv mode
+    int B, I2, O2, L, M, tri, ld_in, ld_out;
+};
+
+int pgemm_launch(int mode, const PgemmArgs& a, int n_work, int64_t ncols_max, hipStream_t s);
+
+// ---- host-side table construction (tables.cpp) -----------------------------------------
+int quadrature(int grid, int nlat, double* theta, double* w);
+// rows l = m..lmax-1 of order m at all latitudes: out[(l-m)*nlat + k]
+struct LegendreGen {
+    int nlat, lmax, mmax, norm, inverse, csphase;
+    std::vector<double> cost;
+    std::vector<double> diag;      // [mmax][nlat]  Pbar_m^m
+    LegendreGen(int mmax, int lmax, int nlat, const double* theta, int norm, int inverse, int csphase);
+    void rows_for_m(int m, double* out) const;
+};
+// packed analysis (weights = P*w) or synthesis (P) streams, and the per-batch block offsets
+void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+                   std::vector<int64_t>& aoff);
+// XCD-aware work list: cost[b] = relative time of one workgroup of batch b, nrb[b] = row blocks
+void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work);
+
+// ---- FFT (fft.hip) -----------------------------------------------------------------------
+struct FftPlan {
+    int n = 0;                     // transform length (nlon)
+    int npass = 0;
+    int radix[24];
+    float2* d_tw = nullptr;        // [n] exp(-2 pi i j / n)
+};
+int fft_plan_init(FftPlan& p, int n);
+void fft_plan_free(FftPlan& p);
+// x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon
+int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+// xm [mmax][nlat][ld] -> x [rows][nlat][nlon]
+int irfft_launch(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+
+// ---- layout passes (layout.hip) ----------------------------------------------------------
+int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri,
+                              hipStream_t s);
+int spectral_to_coeffs_launch(const float* spec, float2* coeffs, int64_t rows, int lmax, int mmax, int ld, int tri,
+                              hipStream_t s);
+int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, hipStream_t s);
+
+}  // namespace sfno
+
+struct sfno_sht_plan {
+    int nlat, nlon, lmax, mmax, grid, norm, csphase, directions, compute, device;
+    sfno::PgemmTable fwd, inv;
+    sfno::FftPlan fft;
+};
+
+struct sfno_dhconv_weights {
+    int I, O, L, compute, device;
+    int nrb, nc;                   // row blocks (over 2*O) and K chunks (over 2*I) per degree
+    sfno::PgemmTable tab;
+};

@@ -1,0 +1,265 @@
+// Host-side construction of quadrature rules, Legendre tables and their packed MFMA
+// operand streams.  Everything here is float64 until the final cast, like the tables the
+// reference modules precompute in numpy before `.float()`
+// (makani/models/networks/sfnonet.py:536-539).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+#include <thread>
+
+#include "sfno_internal.h"
+
+namespace sfno {
+
+static const double kPi = 3.14159265358979323846264338327950288;
+
+// Legendre polynomial P_n(x) and derivative by the three-term recurrence.
+static void legendre_pn(int n, long double x, long double& p, long double& dp) {
+    long double p0 = 1.0L, p1 = x;
+    if (n == 0) { p = 1.0L; dp = 0.0L; return; }
+    for (int k = 2; k <= n; ++k) {
+        long double pk = ((2 * k - 1) * x * p1 - (k - 1) * p0) / k;
+        p0 = p1;
+        p1 = pk;
+    }
+    p = p1;
+    dp = n * (x * p1 - p0) / (x * x - 1.0L);
+}
+
+static void gauss_legendre(int n, double* x, double* w) {
+    for (int i = 0; i < n; ++i) {
+        // ascending nodes: start from the Chebyshev-like guess for the i-th root from the left
+        long double xi = -cosl((long double)kPi * (i + 0.75L) / (n + 0.5L));
+        long double p, dp;
+        for (int it = 0; it < 100; ++it) {
+            legendre_pn(n, xi, p, dp);
+            long double dx = p / dp;
+            xi -= dx;
+            if (fabsl(dx) < 1e-19L) break;
+        }
+        legendre_pn(n, xi, p, dp);
+        x[i] = (double)xi;
+        w[i] = (double)(2.0L / ((1.0L - xi * xi) * dp * dp));
+    }
+}
+
+static void gauss_lobatto(int n, double* x, double* w) {
+    const int N = n - 1;
+    for (int i = 0; i < n; ++i) {
+        long double xi = -cosl((long double)kPi * i / N);
+        if (i == 0) xi = -1.0L;
+        else if (i == N) xi = 1.0L;
+        else {
+            for (int it = 0; it < 100; ++it) {
+                // Newton on q(x) = P'_N(x): q' from the Legendre ODE (1-x^2) P'' = 2x P' - N(N+1) P
+                long double p, dp;
+                legendre_pn(N, xi, p, dp);
+                long double ddp = (2.0L * xi * dp - (long double)N * (N + 1) * p) / (1.0L - xi * xi);
+                long double dx = dp / ddp;
+                xi -= dx;
+                if (fabsl(dx) < 1e-19L) break;
+            }
+        }
+        long double p, dp;
+        if (i == 0) p = (N % 2) ? -1.0L : 1.0L;
+        else if (i == N) p = 1.0L;
+        else legendre_pn(N, xi, p, dp);
+        x[i] = (double)xi;
+        w[i] = (double)(2.0L / ((long double)N * n * p * p));
+    }
+}
+
+static void clenshaw_curtis(int n, double* x, double* w) {
+    const int N = n - 1;
+    for (int k = 0; k < n; ++k) {
+        double theta = kPi - kPi * k / N;     // x ascending from -1
+        x[k] = std::cos(theta);
+        if (n == 2) { w[k] = 1.0; continue; }
+        long double s = 0.0L;
+        for (int j = 1; j <= N / 2; ++j) {
+            long double b = (2 * j == N) ? 1.0L : 2.0L;
+            s += b / (4.0L * j * j - 1.0L) * cosl(2.0L * j * (long double)theta);
+        }
+        double c = (k == 0 || k == N) ? 1.0 : 2.0;
+        w[k] = (double)(c / N * (1.0L - s));
+    }
+    x[0] = -1.0;
+    x[N] = 1.0;
+}
+
+int quadrature(int grid, int nlat, double* theta, double* w) {
+    if (nlat < 2 || !theta || !w) return SFNO_EINVAL;
+    std::vector<double> x(nlat), ww(nlat);
+    switch (grid) {
+        case SFNO_GRID_LEGENDRE_GAUSS: gauss_legendre(nlat, x.data(), ww.data()); break;
+        case SFNO_GRID_LOBATTO: gauss_lobatto(nlat, x.data(), ww.data()); break;
+        case SFNO_GRID_EQUIANGULAR: clenshaw_curtis(nlat, x.data(), ww.data()); break;
+        default: return SFNO_EINVAL;
+    }
+    // x ascends from -1, so arccos descends from pi; flip to north-first (theta ascending)
+    for (int k = 0; k < nlat; ++k) {
+        double xv = std::min(1.0, std::max(-1.0, x[nlat - 1 - k]));
+        theta[k] = std::acos(xv);
+        w[k] = ww[nlat - 1 - k];
+    }
+    return SFNO_OK;
+}
+
+LegendreGen::LegendreGen(int mmax_, int lmax_, int nlat_, const double* theta, int norm_, int inverse_, int csphase_)
+    : nlat(nlat_), lmax(lmax_), mmax(mmax_), norm(norm_), inverse(inverse_), csphase(csphase_) {
+    cost.resize(nlat);
+    for (int k = 0; k < nlat; ++k) cost[k] = std::cos(theta[k]);
+    double nf = (norm == SFNO_NORM_ORTHO) ? 1.0 : std::sqrt(4.0 * kPi);
+    if (inverse) nf = 1.0 / nf;
+    diag.assign((size_t)mmax * nlat, 0.0);
+    for (int k = 0; k < nlat; ++k) diag[k] = nf / std::sqrt(4.0 * kPi);
+    for (int m = 1; m < mmax; ++m)
+        for (int k = 0; k < nlat; ++k) {
+            double c = cost[k];
+            diag[(size_t)m * nlat + k] = std::sqrt((2.0 * m + 1.0) * (1.0 + c) * (1.0 - c) / 2.0 / m) * diag[(size_t)(m - 1) * nlat + k];
+        }
+}
+
+void LegendreGen::rows_for_m(int m, double* out) const {
+    const int nl = lmax - m;
+    if (nl <= 0) return;
+    const double* d = &diag[(size_t)m * nlat];
+    for (int k = 0; k < nlat; ++k) out[k] = d[k];
+    if (nl > 1) {
+        const double f = std::sqrt(2.0 * (m + 1) + 1.0);
+        for (int k = 0; k < nlat; ++k) out[nlat + k] = f * cost[k] * d[k];
+    }
+    for (int l = m + 2; l < lmax; ++l) {
+        const double dl = l, dm = m;
+        const double a = std::sqrt((2 * dl - 1) / (dl - dm) * (2 * dl + 1) / (dl + dm));
+        const double b = std::sqrt((dl + dm - 1) / (dl - dm) * (2 * dl + 1) / (2 * dl - 3) * (dl - dm - 1) / (dl + dm));
+        double* o = out + (size_t)(l - m) * nlat;
+        const double* p1 = o - nlat;
+        const double* p2 = o - 2 * (size_t)nlat;
+        for (int k = 0; k < nlat; ++k) o[k] = cost[k] * a * p1[k] - b * p2[k];
+    }
+    const double sgn = (csphase && (m & 1)) ? -1.0 : 1.0;
+    for (int l = m; l < lmax; ++l) {
+        double f = sgn;
+        if (norm == SFNO_NORM_SCHMIDT) f *= inverse ? std::sqrt(2.0 * l + 1.0) : 1.0 / std::sqrt(2.0 * l + 1.0);
+        if (f != 1.0) {
+            double* o = out + (size_t)(l - m) * nlat;
+            for (int k = 0; k < nlat; ++k) o[k] *= f;
+        }
+    }
+}
+
+static int hw_threads() {
+    unsigned n = std::thread::hardware_concurrency();
+    if (n == 0) n = 4;
+    return (int)std::min(16u, n);
+}
+
+template <class F>
+static void parallel_for(int n, F f) {
+    int nt = std::min(hw_threads(), std::max(1, n));
+    std::vector<std::thread> th;
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([=]() {
+            for (int i = t; i < n; i += nt) f(i);
+        });
+    for (auto& x : th) x.join();
+}
+
+// Packs P (rows x K, accessed through get(row,k)) into the fragment stream described in
+// sfno_internal.h.  dst has nrb*nc blocks.
+template <class G>
+static void pack_blocks(float* dst, int rows, int K, G get) {
+    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
+    for (int rb = 0; rb < nrb; ++rb)
+        for (int c = 0; c < nc; ++c) {
+            float* blk = dst + ((size_t)rb * nc + c) * PG_BLOCK_FLOATS;
+            for (int h = 0; h < 2; ++h)
+                for (int j = 0; j < 64; ++j)
+                    for (int s = 0; s < 4; ++s) {
+                        int row = PG_ROWS * rb + (j & 31);
+                        int k = PG_KC * c + 8 * h + 2 * s + (j >> 5);
+                        float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
+                        blk[(h * 64 + j) * 4 + s] = v;
+                    }
+        }
+}
+
+void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+                   std::vector<int64_t>& aoff) {
+    const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
+    aoff.assign(mmax, 0);
+    int64_t tot = 0;
+    for (int m = 0; m < mmax; ++m) {
+        aoff[m] = tot;
+        int nl = std::max(0, lmax - m);
+        int64_t nrb = analysis ? (nl + PG_ROWS - 1) / PG_ROWS : (nlat + PG_ROWS - 1) / PG_ROWS;
+        int64_t nc = analysis ? (nlat + PG_KC - 1) / PG_KC : (nl + PG_KC - 1) / PG_KC;
+        tot += nrb * nc;
+    }
+    packed.assign((size_t)tot * PG_BLOCK_FLOATS, 0.0f);
+    float* base = packed.data();
+    parallel_for(mmax, [&, base](int m) {
+        int nl = lmax - m;
+        if (nl <= 0) return;
+        std::vector<double> rows((size_t)nl * nlat);
+        g.rows_for_m(m, rows.data());
+        float* dst = base + (size_t)aoff[m] * PG_BLOCK_FLOATS;
+        const double* r = rows.data();
+        if (analysis) {
+            // rows = l - m, K = latitude; value = P * w_k
+            pack_blocks(dst, nl, nlat, [=](int row, int k) { return r[(size_t)row * nlat + k] * quad_w[k]; });
+        } else {
+            // rows = latitude, K = l - m
+            pack_blocks(dst, nlat, nl, [=](int row, int k) { return r[(size_t)k * nlat + row]; });
+        }
+    });
+}
+
+void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work) {
+    // Workgroups are handed to the 8 XCDs round-robin by linear id, so entry 8*i + x of the
+    // list runs on XCD x.  All workgroups of one batch share their Q panel through that XCD's
+    // L2, so a batch is never split across queues; batches are assigned longest-first to the
+    // least loaded queue and each queue runs its batches in decreasing cost order.
+    const int nb = (int)nrb.size();
+    std::vector<int> order(nb);
+    std::iota(order.begin(), order.end(), 0);
+    auto total = [&](int b) { return cost[b] * ((nrb[b] + PG_WAVES - 1) / PG_WAVES); };
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return total(a) > total(b); });
+    std::vector<std::vector<int2>> q(8);
+    double load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int b : order) {
+        if (nrb[b] <= 0) continue;
+        int best = 0;
+        for (int x = 1; x < 8; ++x)
+            if (load[x] < load[best]) best = x;
+        for (int rb = 0; rb < nrb[b]; rb += PG_WAVES) q[best].push_back(make_int2(b, rb));
+        load[best] += total(b);
+    }
+    size_t len = 0;
+    for (auto& v : q) len = std::max(len, v.size());
+    work.assign(len * 8, make_int2(-1, 0));
+    for (int x = 0; x < 8; ++x)
+        for (size_t i = 0; i < q[x].size(); ++i) work[i * 8 + x] = q[x][i];
+}
+
+}  // namespace sfno
+
+extern "C" int sfno_quadrature(int grid, int nlat, double* theta, double* w) {
+    return sfno::quadrature(grid, nlat, theta, w);
+}
+
+extern "C" int sfno_legendre_table(int mmax, int lmax, int nlat, const double* theta, int norm, int inverse,
+                                   int csphase, double* out) {
+    if (mmax < 1 || lmax < 1 || nlat < 1 || !theta || !out) return SFNO_EINVAL;
+    if (norm < 0 || norm > 2) return SFNO_EINVAL;
+    sfno::LegendreGen g(mmax, lmax, nlat, theta, norm, inverse, csphase);
+    std::memset(out, 0, sizeof(double) * (size_t)mmax * lmax * nlat);
+    std::vector<double> rows((size_t)lmax * nlat);
+    for (int m = 0; m < mmax && m < lmax; ++m) {
+        g.rows_for_m(m, rows.data());
+        std::memcpy(out + ((size_t)m * lmax + m) * nlat, rows.data(), sizeof(double) * (size_t)(lmax - m) * nlat);
+    }
+    return SFNO_OK;
+}

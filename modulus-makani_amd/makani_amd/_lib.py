@@ -1,0 +1,68 @@
+"""ctypes binding of libsfno_spectral.so (the C ABI declared in include/sfno_spectral.h).
+
+The library is built in-tree next to this file by ``build.py`` (hipcc, gfx950).  There is
+no fallback implementation: if the shared object is missing, importing this module
+raises, and every compute entry point raises on a non-zero return code.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsfno_spectral.so")
+
+GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2}
+NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
+DIR_FORWARD, DIR_INVERSE = 1, 2
+COMPUTE_FP32, COMPUTE_BF16 = 0, 1
+
+
+class SfnoError(RuntimeError):
+    pass
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build the HIP library first (python modulus-makani_amd/build.py); "
+            "this package has no CPU or PyTorch fallback"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    c = ctypes
+    vp, i32, i64, sz = c.c_void_p, c.c_int, c.c_int64, c.c_size_t
+    dp = c.POINTER(c.c_double)
+    sig = {
+        "sfno_strerror": (c.c_char_p, [i32]),
+        "sfno_version": (i32, []),
+        "sfno_quadrature": (i32, [i32, i32, dp, dp]),
+        "sfno_legendre_table": (i32, [i32, i32, i32, dp, i32, i32, i32, dp]),
+        "sfno_sht_plan_create": (i32, [i32, i32, i32, i32, i32, i32, i32, i32, i32, c.POINTER(vp)]),
+        "sfno_sht_plan_destroy": (i32, [vp]),
+        "sfno_spectral_ld": (i64, [i64]),
+        "sfno_spectral_elems": (i64, [vp, i64]),
+        "sfno_sht_workspace_bytes": (sz, [vp, i64]),
+        "sfno_sht_forward": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_inverse": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_analysis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_synthesis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_coeffs_to_spectral": (i32, [vp, vp, i64, i32, i32, i32, vp]),
+        "sfno_spectral_to_coeffs": (i32, [vp, vp, i64, i32, i32, i32, vp]),
+        "sfno_dhconv_weights_create": (i32, [i32, i32, i32, i32, c.POINTER(vp)]),
+        "sfno_dhconv_weights_update": (i32, [vp, vp, vp]),
+        "sfno_dhconv_weights_destroy": (i32, [vp]),
+        "sfno_dhconv_spectral": (i32, [vp, vp, vp, i32, i32, i32, vp]),
+        "sfno_dhconv_workspace_bytes": (sz, [vp, i32, i32]),
+        "sfno_dhconv": (i32, [vp, vp, vp, i32, i32, i32, vp, sz, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib, tuple(sig)
+
+
+lib, EXPORTS = _load()
+
+
+def check(code, what):
+    if code != 0:
+        raise SfnoError(f"{what} failed: {lib.sfno_strerror(code).decode()} ({code})")

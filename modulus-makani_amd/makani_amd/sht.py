@@ -1,0 +1,231 @@
+"""RealSHT / InverseRealSHT with the torch-harmonics module interface, running on the
+hand-written HIP kernels of libsfno_spectral (gfx950).
+
+Drop-in for the objects Makani builds at makani/models/networks/sfnonet.py:524-539
+(``sht_handle(nlat, nlon, lmax=, mmax=, grid=).float()``) and calls at
+makani/models/common/spectral_convolution.py:131,133,141 and sfnonet.py:596,598,616:
+same constructor arguments, same ``nlat/nlon/lmax/mmax/grid/norm/csphase`` attributes,
+``forward`` maps real ``[..., nlat, nlon]`` to complex ``[..., lmax, mmax]`` and back.
+The Legendre tables live inside a device plan (packed, triangular), not in module
+buffers, so the modules add nothing to a state_dict -- like the non-persistent buffers
+of the reference modules.
+"""
+import ctypes
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from . import _lib
+from ._lib import lib, check
+
+
+def quadrature(grid, nlat):
+    """(theta ascending, weights) of a latitude grid, float64 numpy, from the library's host code."""
+    theta = np.empty(nlat, dtype=np.float64)
+    w = np.empty(nlat, dtype=np.float64)
+    dp = ctypes.POINTER(ctypes.c_double)
+    check(lib.sfno_quadrature(_lib.GRID[grid], nlat, theta.ctypes.data_as(dp), w.ctypes.data_as(dp)), "sfno_quadrature")
+    return theta, w
+
+
+def legendre_gauss_weights(n, a=-1.0, b=1.0):
+    """(cos(theta) ascending, weights) as torch_harmonics.quadrature.legendre_gauss_weights returns them."""
+    theta, w = quadrature("legendre-gauss", n)
+    x = np.cos(theta)[::-1].copy()
+    return (b - a) * 0.5 * x + (b + a) * 0.5, w[::-1].copy() * (b - a) * 0.5
+
+
+def clenshaw_curtiss_weights(n, a=-1.0, b=1.0):
+    theta, w = quadrature("equiangular", n)
+    x = np.cos(theta)[::-1].copy()
+    return (b - a) * 0.5 * x + (b + a) * 0.5, w[::-1].copy() * (b - a) * 0.5
+
+
+def lobatto_weights(n, a=-1.0, b=1.0):
+    theta, w = quadrature("lobatto", n)
+    x = np.cos(theta)[::-1].copy()
+    return (b - a) * 0.5 * x + (b + a) * 0.5, w[::-1].copy() * (b - a) * 0.5
+
+
+def legendre_table(mmax, lmax, theta, norm="ortho", inverse=False, csphase=True):
+    """Dense float64 table [mmax, lmax, nlat] from the library's host recursion."""
+    theta = np.ascontiguousarray(theta, dtype=np.float64)
+    out = np.empty((mmax, lmax, len(theta)), dtype=np.float64)
+    dp = ctypes.POINTER(ctypes.c_double)
+    check(
+        lib.sfno_legendre_table(mmax, lmax, len(theta), theta.ctypes.data_as(dp), _lib.NORM[norm], int(inverse), int(csphase), out.ctypes.data_as(dp)),
+        "sfno_legendre_table",
+    )
+    return out
+
+
+class _Plan:
+    """Owns one sfno_sht_plan on one device."""
+
+    def __init__(self, mod, device, directions):
+        self.handle = ctypes.c_void_p()
+        with torch.cuda.device(device):
+            check(
+                lib.sfno_sht_plan_create(
+                    mod.nlat, mod.nlon, mod.lmax, mod.mmax, _lib.GRID[mod.grid], _lib.NORM[mod.norm], int(mod.csphase), directions,
+                    _lib.COMPUTE_FP32, ctypes.byref(self.handle),
+                ),
+                "sfno_sht_plan_create",
+            )
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib.sfno_sht_plan_destroy(self.handle)
+            self.handle = None
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+class _SHTBase(nn.Module):
+    _directions = 0
+
+    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True):
+        super().__init__()
+        self.nlat = nlat
+        self.nlon = nlon
+        self.grid = grid
+        self.norm = norm
+        self.csphase = csphase
+        if grid == "legendre-gauss" or grid == "equiangular":
+            self.lmax = lmax or self.nlat
+        elif grid == "lobatto":
+            self.lmax = lmax or self.nlat - 1
+        else:
+            raise ValueError("Unknown quadrature mode")
+        if norm not in _lib.NORM:
+            raise ValueError("Unknown normalization mode")
+        self.mmax = mmax or self.nlon // 2 + 1
+        if self.mmax > self.nlon // 2 + 1:
+            raise ValueError("mmax must not exceed nlon // 2 + 1")
+        self._plans = {}
+
+    def extra_repr(self):
+        return f"nlat={self.nlat}, nlon={self.nlon},\n lmax={self.lmax}, mmax={self.mmax},\n grid={self.grid}, csphase={self.csphase}"
+
+    def plan(self, device):
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise RuntimeError("the SFNO spectral kernels run on a HIP device only; move the input to the GPU")
+        key = device.index if device.index is not None else torch.cuda.current_device()
+        p = self._plans.get(key)
+        if p is None:
+            p = _Plan(self, torch.device("cuda", key), self._directions)
+            self._plans[key] = p
+        return p
+
+    def workspace(self, plan, rows, device):
+        nbytes = lib.sfno_sht_workspace_bytes(plan.handle, rows)
+        return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+    def spectral_shape(self, rows):
+        return (self.mmax, self.lmax, int(lib.sfno_spectral_ld(rows)))
+
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state["_plans"] = {}
+        return state
+
+    def __deepcopy__(self, memo):
+        return type(self)(self.nlat, self.nlon, self.lmax, self.mmax, self.grid, self.norm, self.csphase)
+
+
+def _as_fp32_rows(x, tail):
+    if x.is_complex() != (tail == "coeffs"):
+        raise TypeError("expected a real field" if tail == "grid" else "expected complex coefficients")
+    if tail == "grid":
+        if x.dtype in (torch.float16, torch.bfloat16):
+            x = x.float()
+        if x.dtype != torch.float32:
+            raise TypeError(f"the HIP transform computes in float32; got {x.dtype}")
+    else:
+        if x.dtype != torch.complex64:
+            raise TypeError(f"the HIP transform computes in complex64; got {x.dtype}")
+    if x.requires_grad and torch.is_grad_enabled():
+        raise NotImplementedError("backward through the HIP spherical harmonic transforms is not implemented")
+    return x.contiguous()
+
+
+class RealSHT(_SHTBase):
+    """Forward real spherical harmonic transform (analysis)."""
+
+    _directions = _lib.DIR_FORWARD
+
+    @property
+    def weights(self):
+        """Dense analysis table [mmax, lmax, nlat] (float32), as the reference module's buffer of that name."""
+        theta, w = quadrature(self.grid, self.nlat)
+        return torch.from_numpy(legendre_table(self.mmax, self.lmax, theta, self.norm, False, self.csphase) * w).float()
+
+    def forward(self, x):
+        assert x.shape[-2] == self.nlat
+        assert x.shape[-1] == self.nlon
+        x = _as_fp32_rows(x, "grid")
+        lead = x.shape[:-2]
+        rows = int(np.prod(lead)) if len(lead) else 1
+        out = torch.empty((*lead, self.lmax, self.mmax), dtype=torch.complex64, device=x.device)
+        if rows == 0:
+            return out
+        plan = self.plan(x.device)
+        ws, nbytes = self.workspace(plan, rows, x.device)
+        check(lib.sfno_sht_forward(plan.handle, _ptr(x), _ptr(out), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_forward")
+        return out
+
+    def analysis(self, x):
+        """x [..., nlat, nlon] -> spectral-layout float32 [mmax, lmax, ld] (internal fast path)."""
+        assert x.shape[-2] == self.nlat
+        assert x.shape[-1] == self.nlon
+        x = _as_fp32_rows(x, "grid")
+        rows = int(np.prod(x.shape[:-2])) if x.dim() > 2 else 1
+        plan = self.plan(x.device)
+        spec = torch.empty(self.spectral_shape(rows), dtype=torch.float32, device=x.device)
+        ws, nbytes = self.workspace(plan, rows, x.device)
+        check(lib.sfno_sht_analysis(plan.handle, _ptr(x), _ptr(spec), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_analysis")
+        return spec
+
+
+class InverseRealSHT(_SHTBase):
+    """Inverse real spherical harmonic transform (synthesis)."""
+
+    _directions = _lib.DIR_INVERSE
+
+    @property
+    def pct(self):
+        """Dense synthesis table [mmax, lmax, nlat] (float32), as the reference module's buffer of that name."""
+        theta, _ = quadrature(self.grid, self.nlat)
+        return torch.from_numpy(legendre_table(self.mmax, self.lmax, theta, self.norm, True, self.csphase)).float()
+
+    def forward(self, x):
+        assert x.shape[-2] == self.lmax
+        assert x.shape[-1] == self.mmax
+        x = _as_fp32_rows(x, "coeffs")
+        lead = x.shape[:-2]
+        rows = int(np.prod(lead)) if len(lead) else 1
+        out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.float32, device=x.device)
+        if rows == 0:
+            return out
+        plan = self.plan(x.device)
+        ws, nbytes = self.workspace(plan, rows, x.device)
+        check(lib.sfno_sht_inverse(plan.handle, _ptr(x), _ptr(out), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_inverse")
+        return out
+
+    def synthesis(self, spec, lead):
+        """spectral-layout float32 [mmax, lmax, ld] -> x [*lead, nlat, nlon] (internal fast path)."""
+        rows = int(np.prod(lead)) if len(lead) else 1
+        assert tuple(spec.shape) == self.spectral_shape(rows) and spec.dtype == torch.float32 and spec.is_contiguous()
+        plan = self.plan(spec.device)
+        out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.float32, device=spec.device)
+        ws, nbytes = self.workspace(plan, rows, spec.device)
+        check(lib.sfno_sht_synthesis(plan.handle, _ptr(spec), _ptr(out), rows, _ptr(ws), nbytes, _stream_ptr(spec.device)), "sfno_sht_synthesis")
+        return out

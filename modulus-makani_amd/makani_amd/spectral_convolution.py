@@ -1,0 +1,96 @@
+"""SpectralConv with the interface of makani/models/common/spectral_convolution.py:43-148,
+running the forward transform, the dhconv channel mix and the inverse transform on the
+HIP kernels without leaving the order-major spectral layout in between.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from .contractions import get_contract_fun, dhconv_spectral
+from .sht import RealSHT, InverseRealSHT
+
+
+class SpectralConv(nn.Module):
+    """Spectral convolution on the sphere: SHT -> per-degree complex channel mix -> inverse SHT."""
+
+    def __init__(self, forward_transform, inverse_transform, in_channels, out_channels, operator_type="diagonal", separable=False, bias=False, gain=1.0):
+        super().__init__()
+        self.forward_transform = forward_transform
+        self.inverse_transform = inverse_transform
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.modes_lat = self.inverse_transform.lmax
+        self.modes_lon = self.inverse_transform.mmax
+        self.scale_residual = (self.forward_transform.nlat != self.inverse_transform.nlat) or (self.forward_transform.nlon != self.inverse_transform.nlon)
+        if hasattr(self.forward_transform, "grid"):
+            self.scale_residual = self.scale_residual or (self.forward_transform.grid != self.inverse_transform.grid)
+        self.operator_type = operator_type
+        self.separable = separable
+        assert self.inverse_transform.lmax == self.modes_lat
+        assert self.inverse_transform.mmax == self.modes_lon
+
+        weight_shape = [in_channels]
+        if not self.separable:
+            weight_shape += [out_channels]
+        self.modes_lat_local = self.modes_lat
+        self.modes_lon_local = self.modes_lon
+        self.nlat_local = self.inverse_transform.nlat
+        self.nlon_local = self.inverse_transform.nlon
+        if self.operator_type == "diagonal":
+            weight_shape += [self.modes_lat_local, self.modes_lon_local]
+        elif self.operator_type == "dhconv":
+            weight_shape += [self.modes_lat_local]
+        else:
+            raise ValueError(f"Unsupported operator type f{self.operator_type}")
+        if self.operator_type != "dhconv" or self.separable:
+            raise NotImplementedError("the HIP path implements the non-separable 'dhconv' operator")
+
+        # same initialisation as the reference (spectral_convolution.py:97-102)
+        scale = math.sqrt(gain / in_channels) * torch.ones(self.modes_lat_local, dtype=torch.complex64)
+        scale[0] *= math.sqrt(2.0)
+        init = scale * torch.randn(*weight_shape, dtype=torch.complex64)
+        self.weight = nn.Parameter(init)
+
+        self._contract = get_contract_fun(self.weight, implementation="factorized", separable=separable, complex=True, operator_type=operator_type)
+
+        if bias == "constant":
+            self.bias = nn.Parameter(torch.zeros(1, self.out_channels, 1, 1))
+        elif bias == "position":
+            self.bias = nn.Parameter(torch.zeros(1, self.out_channels, self.nlat_local, self.nlon_local))
+
+        self._fused = (
+            isinstance(forward_transform, RealSHT)
+            and isinstance(inverse_transform, InverseRealSHT)
+            and forward_transform.lmax == inverse_transform.lmax
+            and forward_transform.mmax == inverse_transform.mmax
+        )
+
+    def forward(self, x):
+        dtype = x.dtype
+        residual = x
+        x = x.float()
+        B, C, H, W = x.shape
+
+        if self._fused:
+            # the transforms and the contraction all work on float32 regardless of autocast
+            spec = self.forward_transform.analysis(x)
+            if self.scale_residual:
+                residual = self.inverse_transform.synthesis(spec, (B, C)).to(dtype)
+            spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=True)
+            x = self.inverse_transform.synthesis(spec, (B, self.out_channels))
+        else:
+            with torch.autocast(device_type="cuda", enabled=False):
+                x = self.forward_transform(x).contiguous()
+                if self.scale_residual:
+                    residual = self.inverse_transform(x)
+                    residual = residual.to(dtype)
+            xp = self._contract(x, self.weight, separable=self.separable, operator_type=self.operator_type)
+            x = xp.contiguous()
+            with torch.autocast(device_type="cuda", enabled=False):
+                x = self.inverse_transform(x)
+
+        if hasattr(self, "bias"):
+            x = x + self.bias
+        x = x.to(dtype=dtype)
+        return x, residual

@@ -1,0 +1,39 @@
+"""Per-degree complex channel contraction and the SpectralConv op order (oracle).
+
+dhconv restates makani/models/common/contractions.py:130-136
+(einsum "bixy,iox->boxy" on complex tensors); spectral_conv restates the
+orchestration of makani/models/common/spectral_convolution.py:124-148 for the
+non-separable dhconv operator without bias.
+"""
+import numpy as np
+
+from .sht import sht_forward, sht_inverse
+
+
+def dhconv(x, w):
+    """y[b,o,l,m] = sum_i x[b,i,l,m] * w[i,o,l]."""
+    x = np.asarray(x)
+    w = np.asarray(w)
+    assert x.shape[1] == w.shape[0] and x.shape[2] == w.shape[2]
+    return np.einsum("bixy,iox->boxy", x, w, optimize=True)
+
+
+def spectral_conv(x, w, fwd_tables, inv_tables, bias=None):
+    """Returns (y, residual) as SpectralConv.forward does, all in float64.
+
+    residual is the input itself unless the forward and inverse grids differ
+    (spectral_convolution.py:62-64), in which case it is the inverse transform of the
+    unfiltered coefficients (spectral_convolution.py:132-134).
+    """
+    scale_residual = (
+        fwd_tables.nlat != inv_tables.nlat or fwd_tables.nlon != inv_tables.nlon or fwd_tables.grid != inv_tables.grid
+    )
+    residual = np.asarray(x, dtype=np.float64)
+    c = sht_forward(x, fwd_tables)
+    if scale_residual:
+        residual = sht_inverse(c, inv_tables)
+    y = dhconv(c, np.asarray(w, dtype=np.complex128))
+    y = sht_inverse(y, inv_tables)
+    if bias is not None:
+        y = y + bias
+    return y, residual

@@ -42,17 +42,21 @@ class PackedWeights:
             self.handle = None
 
 
-_cache = weakref.WeakKeyDictionary()
+# id(tensor) -> (weak reference to the tensor, PackedWeights); tensors compare element-wise,
+# so they cannot key a WeakKeyDictionary directly
+_cache = {}
 
 
 def packed_for(weight):
     """Packed handle for a weight tensor, cached per tensor object and refreshed when it changes."""
     if weight.device.type != "cuda":
         raise RuntimeError("the dhconv kernel runs on a HIP device only")
-    p = _cache.get(weight)
+    key = id(weight)
+    hit = _cache.get(key)
+    p = hit[1] if hit is not None and hit[0]() is weight else None
     if p is None or p.device != weight.device or p.shape != tuple(weight.shape):
         p = PackedWeights(weight.shape[0], weight.shape[1], weight.shape[2], weight.device)
-        _cache[weight] = p
+        _cache[key] = (weakref.ref(weight, lambda _, k=key: _cache.pop(k, None)), p)
     return p.refresh(weight)
 
 

@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Benchmark of the SFNO spectral hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block]
+
+Default workload (the configuration the headline metric is quoted on): forward + inverse
+real SHT at 721x1440 (equiangular, lmax = mmax = 721), batch 1, 73 channels, float32,
+through the reference-layout module interface (RealSHT.forward then
+InverseRealSHT.forward).  One step = one such pair with the input already resident in
+HBM.  Prints ONE JSON line; `roofline` describes the dominant kernel (the Legendre
+contraction) from HIP-event timings taken in this run, `cpu_baseline` is the PyTorch-CPU
+restatement of the reference op sequence timed on this host on a channel sample.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "modulus-makani_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-channels", type=int, default=4)
+    return ap.parse_args()
+
+
+def event_time_ms(fn, iters, stream):
+    """Average duration of fn() over `iters` launches, HIP events on the launch stream."""
+    import torch
+
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    fn()
+    torch.cuda.synchronize()
+    start.record(stream)
+    for _ in range(iters):
+        fn()
+    stop.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def triangular_count(lmax, mmax):
+    return sum(max(0, lmax - m) for m in range(mmax))
+
+
+def make_fields(isht, channels, device):
+    """Band-limited Gaussian random fields: spectral coefficients with ~l^-2 power, unit variance per channel."""
+    import torch
+
+    lmax, mmax = isht.lmax, isht.mmax
+    coeffs = torch.zeros(1, channels, lmax, mmax, dtype=torch.complex64)
+    scale = 1.0 / (torch.arange(lmax, dtype=torch.float32) + 1.0)
+    tri = torch.tril(torch.ones(lmax, mmax))          # m <= l
+    for c in range(channels):
+        g = torch.Generator().manual_seed(1000 + c)
+        a = torch.complex(torch.randn(lmax, mmax, generator=g), torch.randn(lmax, mmax, generator=g)) / (2.0 ** 0.5)
+        a = a * scale[:, None] * tri
+        a[:, 0] = a[:, 0].real.to(torch.complex64)
+        if mmax == isht.nlon // 2 + 1:
+            a[:, -1] = 0
+        coeffs[0, c] = a
+    x = isht(coeffs.to(device))
+    x = x - x.mean(dim=(-2, -1), keepdim=True)
+    x = x / x.std(dim=(-2, -1), keepdim=True)
+    return x.contiguous()
+
+
+def read_traffic(key):
+    """HBM bytes per launch from the committed rocprofv3 counter summary, if one exists."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
+
+def cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, channels, sample):
+    """Times the reference op sequence (dense fp32 tables, torch.fft + torch.einsum) on the host cores."""
+    import torch
+    from oracle.torch_ref import TorchRefSHT
+
+    torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 1) <= 64 else 64)
+    ref = TorchRefSHT(nlat, nlon, lmax, mmax, grid)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(1, sample, nlat, nlon, generator=g)
+    times = []
+    for it in range(4):
+        t0 = time.perf_counter()
+        y = ref.inverse(ref.forward(x))
+        dt = time.perf_counter() - t0
+        if it:
+            times.append(dt)
+    t = min(times)
+    assert y.shape == x.shape
+    # the pair is linear in the number of channels: scale the sample to the full workload
+    return {
+        "value": (1.0 / t) * (sample / channels),
+        "unit": "pairs/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{sample} of {channels} channels, full {nlat}x{nlon} grid, all orders, dense fp32 tables; best of 3 after 1 warm-up "
+                  f"({t:.3f} s per sample pair), scaled by {sample}/{channels}",
+    }
+
+
+def bench_sht_pair(args):
+    import torch
+    import makani_amd as ma
+    from makani_amd._lib import lib, check
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    nlat, nlon, lmax, mmax, grid, C = 721, 1440, 721, 721, "equiangular", 73
+    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
+    x = make_fields(isht, C, dev)
+    torch.cuda.synchronize()
+
+    def step():
+        return isht(sht(x))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    assert torch.isfinite(y).all()
+
+    # ---- per-stage timings (HIP events on the launch stream) ----------------------------------
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    rows = C
+    pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
+    xm = torch.empty(lib.sfno_fourier_elems(pf, rows), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, rows), dtype=torch.float32, device=dev)
+    coeffs = torch.empty(1, C, lmax, mmax, dtype=torch.complex64, device=dev)
+    out = torch.empty_like(x)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    stages = {
+        "rfft": lambda: check(lib.sfno_rfft(pf, P(x), P(xm), rows, sp), "rfft"),
+        "legendre_analysis": lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), rows, sp), "legendre_analysis"),
+        "spectral_to_coeffs": lambda: check(lib.sfno_spectral_to_coeffs(P(spec), P(coeffs), rows, lmax, mmax, 1, sp), "to_coeffs"),
+        "coeffs_to_spectral": lambda: check(lib.sfno_coeffs_to_spectral(P(coeffs), P(spec), rows, lmax, mmax, 1, sp), "to_spectral"),
+        "legendre_synthesis": lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), rows, sp), "legendre_synthesis"),
+        "irfft": lambda: check(lib.sfno_irfft(pi, P(xm), P(out), rows, sp), "irfft"),
+    }
+    stage_ms = {}
+    for name, fn in stages.items():      # run in pipeline order so every buffer holds real data
+        stage_ms[name] = event_time_ms(fn, max(5, args.steps), stream)
+
+    T = triangular_count(lmax, mmax)
+    leg_flops = 4.0 * rows * nlat * T                 # 2 flop/MAC, Re and Im
+    dom = max(("legendre_analysis", "legendre_synthesis"), key=lambda k: stage_ms[k])
+    achieved = leg_flops / (stage_ms[dom] * 1e-3) / 1e12
+    fft_bytes = rows * nlat * nlon * 4 + rows * nlat * mmax * 8
+    result = {
+        "metric": "SHT fwd+inv/s @721x1440",
+        "value": args.steps / dt,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: RealSHT + InverseRealSHT, equiangular 721x1440, lmax=mmax=721, batch 1, 73 channels, "
+                        "band-limited Gaussian random fields (l^-2 power, unit variance)",
+            "nlat": nlat, "nlon": nlon, "lmax": lmax, "mmax": mmax, "batch": 1, "channels": C,
+        },
+        "roofline": {
+            "kernel": f"pgemm_kernel ({dom})",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+            "traffic": read_traffic(dom),
+            "algorithmic_flops_per_launch": leg_flops,
+            "avg_launch_ms": stage_ms[dom],
+        },
+        "stages_ms": stage_ms,
+        "fft_hbm": {
+            "rfft_GBps": fft_bytes / (stage_ms["rfft"] * 1e-3) / 1e9,
+            "irfft_GBps": fft_bytes / (stage_ms["irfft"] * 1e-3) / 1e9,
+            "peak_GBps": PEAK_HBM_GBS,
+            "algorithmic_bytes_per_launch": fft_bytes,
+        },
+    }
+    if not args.no_cpu_baseline:
+        del xm, spec, coeffs, out
+        result["cpu_baseline"] = cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, C, args.cpu_sample_channels)
+    return result
+
+
+def bench_spectral_block(args):
+    """configs[2]: forward SHT -> dhconv -> inverse SHT on a 241x480 Legendre-Gauss grid, 384 channels."""
+    import torch
+    import makani_amd as ma
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    nlat, nlon, L, M, C = 241, 480, 241, 241, 384
+    sht = ma.RealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss")
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss")
+    conv = ma.SpectralConv(sht, isht, C, C, operator_type="dhconv").to(dev)
+    g = torch.Generator().manual_seed(3)
+    w = torch.complex(torch.randn(C, C, L, generator=g), torch.randn(C, C, L, generator=g)) / (2.0 ** 0.5) * (1.0 / C) ** 0.5
+    with torch.no_grad():
+        conv.weight.copy_(w.to(dev))
+    x = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(2)).to(dev)
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            conv(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y, _ = conv(x)
+        torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert torch.isfinite(y).all()
+    Tp = sum(min(l + 1, M) for l in range(L))
+    dh_flops = 8.0 * C * C * Tp
+    leg_flops = 4.0 * C * nlat * triangular_count(L, M)
+    return {
+        "metric": "spectral block fwd/s @241x480x384",
+        "value": args.steps / dt,
+        "unit": "blocks/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[2]: SHT -> dhconv -> inverse SHT, legendre-gauss 241x480, lmax=mmax=241, batch 1, 384 channels"},
+        "useful_TFLOPs_per_step": (dh_flops + 2 * leg_flops) / 1e12,
+        "achieved_TFLOPs": (dh_flops + 2 * leg_flops) / (dt / args.steps) / 1e12,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (the spectral path has no multi-GPU part)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(1)
+    res = bench_sht_pair(args) if args.workload == "sht_pair" else bench_spectral_block(args)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

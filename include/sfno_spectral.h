@@ -113,6 +113,19 @@ int sfno_sht_analysis(const sfno_sht_plan* plan, const float* x, float* spec, in
 int sfno_sht_synthesis(const sfno_sht_plan* plan, const float* spec, float* x, int64_t rows,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* The four stages of the transform pair on their own (what sfno_sht_analysis and
+ * sfno_sht_synthesis chain).  xm is the order-major Fourier buffer float32
+ * [mmax][nlat][ld]: (re,im) of 2 pi/nlon * sum_n x[r][k][n] e^{-i m phi_n} at
+ * xm[m][k][2r], xm[m][k][2r+1]. */
+int sfno_rfft(const sfno_sht_plan* plan, const float* x, float* xm, int64_t rows, void* stream);
+int sfno_irfft(const sfno_sht_plan* plan, const float* xm, float* x, int64_t rows, void* stream);
+int sfno_legendre_analysis(const sfno_sht_plan* plan, const float* xm, float* spec, int64_t rows,
+                           void* stream);
+int sfno_legendre_synthesis(const sfno_sht_plan* plan, const float* spec, float* xm, int64_t rows,
+                            void* stream);
+/* floats in one xm buffer: mmax * nlat * ld */
+int64_t sfno_fourier_elems(const sfno_sht_plan* plan, int64_t rows);
+
 /* layout passes between the reference coefficient layout and the spectral layout */
 /* `triangular` != 0: only entries with m <= l are moved (to_coeffs writes zeros for
  * m > l); 0: the whole lmax x mmax rectangle is moved. */

@@ -153,18 +153,46 @@ extern "C" size_t sfno_sht_workspace_bytes(const sfno_sht_plan* p, int64_t rows)
     return carve(p, rows, nullptr).bytes;
 }
 
+extern "C" int64_t sfno_fourier_elems(const sfno_sht_plan* p, int64_t rows) {
+    if (!p || rows <= 0) return 0;
+    return (int64_t)p->mmax * p->nlat * sfno_spectral_ld(rows);
+}
+
+extern "C" int sfno_rfft(const sfno_sht_plan* p, const float* x, float* xm, int64_t rows, void* stream) {
+    if (!p || !x || !xm || !rows_ok(rows)) return SFNO_EINVAL;
+    return rfft_launch(p->fft, x, xm, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+}
+
+extern "C" int sfno_irfft(const sfno_sht_plan* p, const float* xm, float* x, int64_t rows, void* stream) {
+    if (!p || !x || !xm || !rows_ok(rows)) return SFNO_EINVAL;
+    return irfft_launch(p->fft, xm, x, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+}
+
+extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, float* spec, int64_t rows, void* stream) {
+    if (!p || !xm || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
+    const int64_t ld = sfno_spectral_ld(rows);
+    PgemmArgs a = legendre_args(p, p->fwd, xm, spec, ld);
+    return pgemm_launch(PG_ANALYSIS, a, p->fwd.n_work, ld, (hipStream_t)stream);
+}
+
+extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec, float* xm, int64_t rows, void* stream) {
+    if (!p || !xm || !spec || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
+    const int64_t ld = sfno_spectral_ld(rows);
+    PgemmArgs a = legendre_args(p, p->inv, spec, xm, ld);
+    return pgemm_launch(PG_SYNTHESIS, a, p->inv.n_work, ld, (hipStream_t)stream);
+}
+
 extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const float* x, float* spec, int64_t rows, void* workspace,
                                  size_t workspace_bytes, void* stream) {
     if (!p || !x || !spec || !rows_ok(rows)) return SFNO_EINVAL;
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
-    hipStream_t s = (hipStream_t)stream;
-    const int64_t ld = sfno_spectral_ld(rows);
-    int rc = rfft_launch(p->fft, x, w.xm, rows, p->nlat, p->mmax, (int)ld, s);
+    int rc = sfno_rfft(p, x, w.xm, rows, stream);
     if (rc != SFNO_OK) return rc;
-    PgemmArgs a = legendre_args(p, p->fwd, w.xm, spec, ld);
-    return pgemm_launch(PG_ANALYSIS, a, p->fwd.n_work, ld, s);
+    return sfno_legendre_analysis(p, w.xm, spec, rows, stream);
 }
 
 extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, float* x, int64_t rows, void* workspace,
@@ -173,12 +201,9 @@ extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, flo
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
-    hipStream_t s = (hipStream_t)stream;
-    const int64_t ld = sfno_spectral_ld(rows);
-    PgemmArgs a = legendre_args(p, p->inv, spec, w.xm, ld);
-    int rc = pgemm_launch(PG_SYNTHESIS, a, p->inv.n_work, ld, s);
+    int rc = sfno_legendre_synthesis(p, spec, w.xm, rows, stream);
     if (rc != SFNO_OK) return rc;
-    return irfft_launch(p->fft, w.xm, x, rows, p->nlat, p->mmax, (int)ld, s);
+    return sfno_irfft(p, w.xm, x, rows, stream);
 }
 
 extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* coeffs, int64_t rows, void* workspace,

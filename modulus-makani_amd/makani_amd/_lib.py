@@ -44,6 +44,11 @@ def _load():
         "sfno_sht_inverse": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_analysis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_synthesis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_rfft": (i32, [vp, vp, vp, i64, vp]),
+        "sfno_irfft": (i32, [vp, vp, vp, i64, vp]),
+        "sfno_legendre_analysis": (i32, [vp, vp, vp, i64, vp]),
+        "sfno_legendre_synthesis": (i32, [vp, vp, vp, i64, vp]),
+        "sfno_fourier_elems": (i64, [vp, i64]),
         "sfno_coeffs_to_spectral": (i32, [vp, vp, i64, i32, i32, i32, vp]),
         "sfno_spectral_to_coeffs": (i32, [vp, vp, i64, i32, i32, i32, vp]),
         "sfno_dhconv_weights_create": (i32, [i32, i32, i32, i32, c.POINTER(vp)]),

@@ -13,27 +13,34 @@ with c = cos(theta); Condon-Shortley phase flips odd m.
 import numpy as np
 
 
-def legpoly(mmax, lmax, theta, norm="ortho", inverse=False, csphase=True):
+def legpoly(mmax, lmax, theta, norm="ortho", inverse=False, csphase=True, contiguous=True):
     """Table vdm[m, l, k] = Pbar_l^m(cos theta_k), zero for l < m; float64."""
     theta = np.asarray(theta, dtype=np.float64)
     nmax = max(mmax, lmax)
     c = np.cos(theta)
-    vdm = np.zeros((nmax, nmax, len(theta)), dtype=np.float64)
+    # stored degree-major (v[l, m, k]) so that each recursion step touches contiguous memory;
+    # the returned array is the [m, l, k] view of it
+    v = np.zeros((nmax, nmax, len(theta)), dtype=np.float64)
     norm_factor = 1.0 if norm == "ortho" else np.sqrt(4.0 * np.pi)
     norm_factor = 1.0 / norm_factor if inverse else norm_factor
-    vdm[0, 0, :] = norm_factor / np.sqrt(4.0 * np.pi)
+    v[0, 0, :] = norm_factor / np.sqrt(4.0 * np.pi)
     for l in range(1, nmax):
-        vdm[l - 1, l, :] = np.sqrt(2 * l + 1) * c * vdm[l - 1, l - 1, :]
-        vdm[l, l, :] = np.sqrt((2 * l + 1) * (1 + c) * (1 - c) / 2 / l) * vdm[l - 1, l - 1, :]
+        v[l, l - 1, :] = np.sqrt(2 * l + 1) * c * v[l - 1, l - 1, :]
+        v[l, l, :] = np.sqrt((2 * l + 1) * (1 + c) * (1 - c) / 2 / l) * v[l - 1, l - 1, :]
     for l in range(2, nmax):
         m = np.arange(0, l - 1, dtype=np.float64)
         a = np.sqrt((2 * l - 1) / (l - m) * (2 * l + 1) / (l + m))
         b = np.sqrt((l + m - 1) / (l - m) * (2 * l + 1) / (2 * l - 3) * (l - m - 1) / (l + m))
-        vdm[: l - 1, l, :] = c[None, :] * a[:, None] * vdm[: l - 1, l - 1, :] - b[:, None] * vdm[: l - 1, l - 2, :]
+        # v[l] = c a v[l-1] - b v[l-2], evaluated in place (no full-size temporaries)
+        cur = v[l, : l - 1, :]
+        np.multiply(v[l - 1, : l - 1, :], c[None, :], out=cur)
+        cur *= a[:, None]
+        tmp = v[l - 2, : l - 1, :] * b[:, None]
+        cur -= tmp
     if norm == "schmidt":
         fac = np.sqrt(2.0 * np.arange(nmax) + 1.0)
-        vdm = vdm * fac[None, :, None] if inverse else vdm / fac[None, :, None]
-    vdm = vdm[:mmax, :lmax].copy()
+        v = v * fac[:, None, None] if inverse else v / fac[:, None, None]
+    v = v[:lmax, :mmax]
     if csphase:
-        vdm[1::2] *= -1.0
-    return vdm
+        v[:, 1::2] *= -1.0
+    return np.ascontiguousarray(v.transpose(1, 0, 2)) if contiguous else v.transpose(1, 0, 2)

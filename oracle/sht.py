@@ -27,20 +27,35 @@ class ShtTables:
         self.mmax = mmax or nlon // 2 + 1
         self._weights = None
         self._pct = None
+        self._pfwd = None
 
     @property
     def weights(self):
         """Analysis table [m, l, k] (Legendre * quadrature weight)."""
         if self._weights is None:
-            p = legpoly(self.mmax, self.lmax, self.theta, norm=self.norm, inverse=False, csphase=self.csphase)
-            self._weights = p * self.quad_w[None, None, :]
+            p = legpoly(self.mmax, self.lmax, self.theta, norm=self.norm, inverse=False, csphase=self.csphase, contiguous=False)
+            p *= self.quad_w[None, None, :]
+            self._weights = p
         return self._weights
+
+    @property
+    def p_analysis(self):
+        """Legendre table of the forward transform without the quadrature weights, [m, l, k].
+
+        For norm="ortho" it equals the synthesis table, which is then shared (the
+        721-point tables are 3 GB each in float64).
+        """
+        if self.norm == "ortho":
+            return self.pct
+        if self._pfwd is None:
+            self._pfwd = legpoly(self.mmax, self.lmax, self.theta, norm=self.norm, inverse=False, csphase=self.csphase, contiguous=False)
+        return self._pfwd
 
     @property
     def pct(self):
         """Synthesis table [m, l, k]."""
         if self._pct is None:
-            self._pct = legpoly(self.mmax, self.lmax, self.theta, norm=self.norm, inverse=True, csphase=self.csphase)
+            self._pct = legpoly(self.mmax, self.lmax, self.theta, norm=self.norm, inverse=True, csphase=self.csphase, contiguous=False)
         return self._pct
 
 
@@ -56,16 +71,35 @@ def irfft_lon(X, nlon):
 
 
 def legendre_analysis(X, weights):
-    """c[..., l, m] = sum_k X[..., k, m] weights[m, l, k] (per-order real contraction on Re and Im)."""
-    # matmul over m: (m, l, k) @ (..., m, k, 1)
-    Xm = np.moveaxis(X, -1, -2)                                # (..., m, k)
-    c = np.einsum("mlk,...mk->...lm", weights, Xm, optimize=True)
-    return c
+    """c[..., l, m] = sum_k X[..., k, m] weights[m, l, k] (per-order real contraction on Re and Im).
+
+    Evaluated as one real matrix product per order m (the einsum '...km,mlk->...lm' of the
+    reference, applied to Re and Im); degrees l < m have zero weights and are skipped.
+    """
+    mmax, lmax, nlat = weights.shape
+    lead = X.shape[:-2]
+    Xf = np.ascontiguousarray(X).reshape(-1, nlat, X.shape[-1])
+    rows = Xf.shape[0]
+    c = np.zeros((rows, lmax, mmax), dtype=np.complex128)
+    for m in range(min(mmax, lmax)):
+        xm = np.ascontiguousarray(Xf[:, :, m])             # (rows, nlat) complex
+        w = np.ascontiguousarray(weights[m, m:, :])        # (lmax-m, nlat) real
+        c[:, m:, m] = (xm.real @ w.T) + 1j * (xm.imag @ w.T)
+    return c.reshape(*lead, lmax, mmax)
 
 
 def legendre_synthesis(c, pct):
     """X[..., k, m] = sum_l c[..., l, m] pct[m, l, k]."""
-    return np.einsum("mlk,...lm->...km", pct, c, optimize=True)
+    mmax, lmax, nlat = pct.shape
+    lead = c.shape[:-2]
+    cf = np.ascontiguousarray(c).reshape(-1, lmax, mmax)
+    rows = cf.shape[0]
+    X = np.zeros((rows, nlat, mmax), dtype=np.complex128)
+    for m in range(min(mmax, lmax)):
+        cm = np.ascontiguousarray(cf[:, m:, m])            # (rows, lmax-m)
+        p = np.ascontiguousarray(pct[m, m:, :])            # (lmax-m, nlat)
+        X[:, :, m] = (cm.real @ p) + 1j * (cm.imag @ p)
+    return X.reshape(*lead, nlat, mmax)
 
 
 def sht_forward(x, tables):
@@ -73,7 +107,8 @@ def sht_forward(x, tables):
     assert x.shape[-2] == tables.nlat
     assert x.shape[-1] == tables.nlon
     X = rfft_lon(x.astype(np.float64), tables.mmax)
-    return legendre_analysis(X, tables.weights)
+    # weights[m, l, k] = P[m, l, k] * w[k]: fold w into X instead of materialising a second table
+    return legendre_analysis(X * tables.quad_w[:, None], tables.p_analysis)
 
 
 def sht_inverse(c, tables):

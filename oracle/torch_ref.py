@@ -1,0 +1,50 @@
+"""PyTorch-CPU float32 restatement of the reference op sequence (oracle; CPU baseline).
+
+This is what the reference executes on a CPU: dense float32 tables held as tensors,
+``torch.fft.rfft`` -> two ``torch.einsum('...km,mlk->...lm')`` -> (dhconv einsum) ->
+two ``torch.einsum('...lm,mlk->...km')`` -> ``torch.fft.irfft`` (torch-harmonics'
+RealSHT / InverseRealSHT forward as called from
+makani/models/common/spectral_convolution.py:131,141, and
+makani/models/common/contractions.py:134).  It is timed by bench.py's cpu_baseline leg
+and never used by the product.
+"""
+import numpy as np
+import torch
+
+from .sht import ShtTables
+
+
+class TorchRefSHT:
+    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, directions=("fwd", "inv")):
+        t = ShtTables(nlat, nlon, lmax, mmax, grid, norm, csphase)
+        self.nlat, self.nlon, self.lmax, self.mmax = nlat, nlon, t.lmax, t.mmax
+        self.weights = None
+        self.pct = None
+        if "inv" in directions:
+            self.pct = torch.from_numpy(np.ascontiguousarray(t.pct.astype(np.float32)))
+        if "fwd" in directions:
+            w = t.p_analysis.astype(np.float32)
+            w *= t.quad_w[None, None, :].astype(np.float32)
+            self.weights = torch.from_numpy(np.ascontiguousarray(w))
+
+    def forward(self, x):
+        x = 2.0 * torch.pi * torch.fft.rfft(x, dim=-1, norm="forward")
+        x = torch.view_as_real(x)
+        out_shape = list(x.size())
+        out_shape[-3] = self.lmax
+        out_shape[-2] = self.mmax
+        xout = torch.zeros(out_shape, dtype=x.dtype)
+        xout[..., 0] = torch.einsum("...km,mlk->...lm", x[..., : self.mmax, 0], self.weights)
+        xout[..., 1] = torch.einsum("...km,mlk->...lm", x[..., : self.mmax, 1], self.weights)
+        return torch.view_as_complex(xout)
+
+    def inverse(self, c):
+        c = torch.view_as_real(c)
+        rl = torch.einsum("...lm,mlk->...km", c[..., 0], self.pct)
+        im = torch.einsum("...lm,mlk->...km", c[..., 1], self.pct)
+        x = torch.view_as_complex(torch.stack((rl, im), -1))
+        return torch.fft.irfft(x, n=self.nlon, dim=-1, norm="forward")
+
+
+def dhconv(x, w):
+    return torch.einsum("bixy,iox->boxy", x, w)

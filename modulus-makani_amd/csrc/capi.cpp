@@ -119,7 +119,9 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if (!out) return SFNO_EINVAL;
     *out = nullptr;
     if (nlat < 2 || nlon < 1 || lmax < 1 || mmax < 1) return SFNO_EINVAL;
-    if (mmax > nlon / 2 + 1) return SFNO_EINVAL;
+    // the forward transform keeps the first mmax of nlon/2+1 Fourier bins; the inverse zero-pads or
+    // drops orders like a C2R transform, so only the forward direction bounds mmax
+    if ((directions & SFNO_DIR_FORWARD) && mmax > nlon / 2 + 1) return SFNO_EINVAL;
     if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
     if (!(directions & (SFNO_DIR_FORWARD | SFNO_DIR_INVERSE))) return SFNO_EINVAL;
     if (compute != SFNO_COMPUTE_FP32) return SFNO_EUNSUPPORTED;

@@ -307,7 +307,8 @@ int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int n
 }
 
 int irfft_launch(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
-    if (mmax > p.n / 2 + 1 || ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
+    // orders above nlon/2 are dropped, as torch.fft.irfft(n=nlon) drops surplus input bins
+    if (ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
     switch (pick_pairs(p.n)) {
         case 4: return irfft_go<4>(p, xm, x, rows, nlat, mmax, ld, s);
         case 2: return irfft_go<2>(p, xm, x, rows, nlat, mmax, ld, s);

@@ -107,8 +107,8 @@ class _SHTBase(nn.Module):
         if norm not in _lib.NORM:
             raise ValueError("Unknown normalization mode")
         self.mmax = mmax or self.nlon // 2 + 1
-        if self.mmax > self.nlon // 2 + 1:
-            raise ValueError("mmax must not exceed nlon // 2 + 1")
+        if (self._directions & _lib.DIR_FORWARD) and self.mmax > self.nlon // 2 + 1:
+            raise ValueError("mmax must not exceed nlon // 2 + 1 for the forward transform")
         self._plans = {}
 
     def extra_repr(self):

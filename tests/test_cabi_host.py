@@ -1,0 +1,101 @@
+"""CPU-side checks of the C ABI library: it loads, exports every declared symbol, and its
+host-only table builders agree with the oracle (no GPU compute is called here)."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle.quadrature import grid_nodes
+from oracle.legendre import legpoly
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sfno_spectral.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sfno_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib_built):
+    import ctypes
+
+    lib = ctypes.CDLL(lib_built)
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), n
+    import makani_amd._lib as L
+
+    assert sorted(L.EXPORTS) == names
+    assert L.lib.sfno_version() >= 1
+    assert L.lib.sfno_strerror(-1).decode() == "invalid argument"
+
+
+@pytest.mark.parametrize("grid", ["legendre-gauss", "lobatto", "equiangular"])
+@pytest.mark.parametrize("nlat", [2, 3, 16, 33, 240, 721])
+def test_quadrature_matches_oracle(lib_built, grid, nlat):
+    import makani_amd as ma
+
+    theta, w = ma.quadrature(grid, nlat)
+    t0, w0 = grid_nodes(nlat, grid)
+    assert np.allclose(theta, t0, atol=1e-13) and np.allclose(w, w0, atol=1e-13)
+    assert abs(w.sum() - 2.0) < 1e-12
+
+
+def test_quadrature_module_functions(lib_built):
+    import makani_amd as ma
+
+    for fn in (ma.legendre_gauss_weights, ma.clenshaw_curtiss_weights, ma.lobatto_weights):
+        x, w = fn(20)
+        assert np.all(np.diff(x) > 0) and abs(w.sum() - 2.0) < 1e-12       # tests/test_metrics.py:37-45
+        x, w = fn(20, a=0.0, b=3.0)
+        assert abs(w.sum() - 3.0) < 1e-12 and x.min() >= 0 and x.max() <= 3
+
+
+@pytest.mark.parametrize("norm", ["ortho", "four-pi", "schmidt"])
+@pytest.mark.parametrize("inverse", [False, True])
+@pytest.mark.parametrize("csphase", [True, False])
+def test_legendre_table_matches_oracle(lib_built, norm, inverse, csphase):
+    import makani_amd as ma
+
+    theta, _ = grid_nodes(40, "equiangular")
+    for mmax, lmax in ((21, 20), (9, 33), (40, 40)):
+        got = ma.legendre_table(mmax, lmax, theta, norm, inverse, csphase)
+        ref = legpoly(mmax, lmax, theta, norm, inverse, csphase)
+        assert np.allclose(got, ref, rtol=1e-11, atol=1e-14)
+
+
+def test_legendre_table_large_orders(lib_built):
+    import makani_amd as ma
+
+    theta, _ = grid_nodes(721, "equiangular")
+    got = ma.legendre_table(721, 721, theta[300:310], "ortho", False, True)
+    ref = legpoly(721, 721, theta[300:310])
+    assert np.isfinite(got).all()
+    assert np.allclose(got, ref, rtol=1e-9, atol=1e-12)
+
+
+def test_module_attributes_and_errors(lib_built):
+    import torch
+    import makani_amd as ma
+
+    s = ma.RealSHT(32, 64, grid="legendre-gauss")
+    assert (s.nlat, s.nlon, s.lmax, s.mmax, s.grid) == (32, 64, 32, 33, "legendre-gauss")
+    assert ma.RealSHT(32, 64).lmax == 31                         # lobatto default
+    assert ma.InverseRealSHT(32, 64, lmax=10, mmax=8, grid="equiangular").mmax == 8
+    assert list(s.state_dict().keys()) == [] and list(s.buffers()) == []
+    s.float()
+    with pytest.raises(ValueError):
+        ma.RealSHT(32, 64, grid="nope")
+    with pytest.raises(RuntimeError):
+        s(torch.zeros(1, 32, 64))                                # CPU tensors are refused: no fallback path
+    w = s.weights
+    assert tuple(w.shape) == (33, 32, 32) and w.dtype == torch.float32
+    conv = ma.SpectralConv(s, ma.InverseRealSHT(32, 64, grid="legendre-gauss"), 4, 6, operator_type="dhconv", gain=2.0)
+    assert tuple(conv.weight.shape) == (4, 6, 32) and conv.weight.dtype == torch.complex64
+    assert not conv.scale_residual
+    assert ma.SpectralConv(s, ma.InverseRealSHT(16, 32, lmax=32, mmax=33, grid="legendre-gauss"), 4, 6, operator_type="dhconv").scale_residual
+    with pytest.raises(ValueError):
+        ma.SpectralConv(s, ma.InverseRealSHT(32, 64, grid="legendre-gauss"), 4, 6, operator_type="bogus")

@@ -113,3 +113,17 @@ def test_shape_asserts(lib_built):
     isht = ma.InverseRealSHT(16, 32, grid="legendre-gauss")
     with pytest.raises(AssertionError):
         isht(torch.zeros(2, 16, 16, dtype=torch.complex64, device="cuda"))
+
+
+def test_inverse_surplus_orders(lib_built):
+    """mmax above nlon//2+1 (up-scaled coefficients synthesised on a coarser grid): surplus orders are dropped like irfft does."""
+    import makani_amd as ma
+
+    t = ShtTables(16, 32, 32, 33, "legendre-gauss")
+    torch.manual_seed(5)
+    c = torch.randn(3, 32, 33, dtype=torch.complex64)
+    got = ma.InverseRealSHT(16, 32, lmax=32, mmax=33, grid="legendre-gauss")(c.cuda())
+    ref = sht_inverse(c.numpy().astype(np.complex128), t)
+    assert rel_l2(got.cpu().numpy(), ref) < TOL
+    with pytest.raises(ValueError):
+        ma.RealSHT(16, 32, lmax=32, mmax=33, grid="legendre-gauss")

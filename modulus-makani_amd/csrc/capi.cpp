@@ -107,7 +107,8 @@ extern "C" const char* sfno_strerror(int code) {
 
 extern "C" int sfno_version(void) { return kVersion; }
 
-extern "C" int64_t sfno_spectral_ld(int64_t rows) { return (2 * rows + 3) / 4 * 4; }
+// 16 floats = 64 bytes: the pieces of a row that FFT workgroups exchange with HBM stay cache-line aligned
+extern "C" int64_t sfno_spectral_ld(int64_t rows) { return (2 * rows + 15) / 16 * 16; }
 
 extern "C" int64_t sfno_spectral_elems(const sfno_sht_plan* p, int64_t rows) {
     if (!p || rows <= 0) return 0;

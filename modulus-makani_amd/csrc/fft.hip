@@ -240,12 +240,14 @@ int fft_plan_init(FftPlan& p, int n) {
     }
     if (hipMalloc(&p.d_tw, sizeof(float2) * n) != hipSuccess) return SFNO_ENOMEM;
     if (hipMemcpy(p.d_tw, tw.data(), sizeof(float2) * n, hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
-    return SFNO_OK;
+    return fft_fast_plan_init(p);
 }
 
 void fft_plan_free(FftPlan& p) {
     if (p.d_tw) (void)hipFree(p.d_tw);
-    p.d_tw = nullptr;
+    if (p.d_tw0) (void)hipFree(p.d_tw0);
+    if (p.d_tw1) (void)hipFree(p.d_tw1);
+    p.d_tw = p.d_tw0 = p.d_tw1 = nullptr;
 }
 
 static FftDev make_dev(const FftPlan& p) {
@@ -298,6 +300,7 @@ static int pick_pairs(int n) {
 
 int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     if (mmax > p.n / 2 + 1 || ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
+    if (fft_fast_supported(p.n)) return fft_fast_launch(false, p, x, xm, rows, nlat, mmax, ld, s);
     switch (pick_pairs(p.n)) {
         case 4: return rfft_go<4>(p, x, xm, rows, nlat, mmax, ld, s);
         case 2: return rfft_go<2>(p, x, xm, rows, nlat, mmax, ld, s);
@@ -309,6 +312,7 @@ int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int n
 int irfft_launch(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     // orders above nlon/2 are dropped, as torch.fft.irfft(n=nlon) drops surplus input bins
     if (ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
+    if (fft_fast_supported(p.n)) return fft_fast_launch(true, p, xm, x, rows, nlat, mmax, ld, s);
     switch (pick_pairs(p.n)) {
         case 4: return irfft_go<4>(p, xm, x, rows, nlat, mmax, ld, s);
         case 2: return irfft_go<2>(p, xm, x, rows, nlat, mmax, ld, s);

@@ -1,0 +1,487 @@
+// Specialised longitude FFTs for the transform lengths the SFNO uses (1440 = 16*10*9,
+// 480 = 10*16*3, ...): everything about the length is a compile-time constant.
+//
+// A workgroup transforms S complex sequences (2*S channels at one latitude) held in LDS.
+// The length factors as N = R0*R1*R2 and every pass is one radix-R butterfly per thread,
+// computed in registers by a compile-time Cooley-Tukey recursion over the base radices
+// 2,3,4,5 with constant twiddles.  Passes work in place:
+//   forward (rfft) : decimation in frequency, natural-order input, digit-reversed output,
+//                    which the Hermitian split / order-major store gathers anyway;
+//   inverse (irfft): decimation in time, the Hermitian extension scatters its input to
+//                    digit-reversed positions, output is in natural order so rows leave
+//                    LDS as contiguous float4 stores.
+// Inter-pass twiddles come from two small per-plan tables (float64-computed, read through
+// L1): tw0[(k0-1)*(N/R0) + j] = w_N^(k0*j), tw1[(k1-1)*R2 + n2] = w_N^(R0*k1*n2).
+#include "sfno_internal.h"
+
+#include <cmath>
+#include <vector>
+
+namespace sfno {
+
+namespace {
+
+constexpr double kTwoPi = 6.283185307179586476925286766559;
+
+constexpr double ct_cos(double x) {
+    double term = 1.0, sum = 1.0;
+    for (int i = 1; i <= 24; ++i) {
+        term *= -x * x / ((2.0 * i - 1.0) * (2.0 * i));
+        sum += term;
+    }
+    return sum;
+}
+constexpr double ct_sin(double x) {
+    double term = x, sum = x;
+    for (int i = 1; i <= 24; ++i) {
+        term *= -x * x / ((2.0 * i) * (2.0 * i + 1.0));
+        sum += term;
+    }
+    return sum;
+}
+
+// forward twiddles w_R^i = exp(-2 pi i / R): c = cos, s = -sin
+template <int R>
+struct TwTab {
+    float c[R];
+    float s[R];
+};
+template <int R>
+constexpr TwTab<R> make_tw() {
+    TwTab<R> t{};
+    for (int i = 0; i < R; ++i) {
+        // reduce to (-pi, pi] for the series; quarter turns are exact
+        int num = i % R;
+        double c = 0.0, s = 0.0;
+        if ((4 * num) % R == 0) {
+            int q = (4 * num) / R;
+            c = (q == 0) ? 1.0 : (q == 2) ? -1.0 : 0.0;
+            s = (q == 1) ? 1.0 : (q == 3) ? -1.0 : 0.0;
+        } else {
+            double x = kTwoPi * (double)num / (double)R;
+            if (x > kTwoPi / 2) x -= kTwoPi;
+            c = ct_cos(x);
+            s = ct_sin(x);
+        }
+        t.c[i] = (float)c;
+        t.s[i] = (float)(-s);
+    }
+    return t;
+}
+
+__device__ __forceinline__ float2 cmul(float2 a, float2 b) { return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x); }
+__device__ __forceinline__ float2 cadd(float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); }
+__device__ __forceinline__ float2 csub(float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); }
+template <int INV>
+__device__ __forceinline__ float2 mul_mi(float2 a) { return INV ? make_float2(-a.y, a.x) : make_float2(a.y, -a.x); }
+template <int INV>
+__device__ __forceinline__ float2 cmul_tw(float2 a, float2 w) {
+    if (INV) w.y = -w.y;
+    return cmul(a, w);
+}
+
+constexpr int first_factor(int r) { return (r % 4 == 0 && r > 4) ? 4 : (r % 2 == 0) ? 2 : (r % 3 == 0) ? 3 : (r % 5 == 0) ? 5 : r; }
+
+// In-register DFT of length R (natural order in and out), sign -1 (INV = 0) or +1 (INV = 1).
+template <int R, int INV>
+__device__ __forceinline__ void dft(float2 (&v)[R]) {
+    if constexpr (R == 1) {
+    } else if constexpr (R == 2) {
+        float2 a = v[0], b = v[1];
+        v[0] = cadd(a, b);
+        v[1] = csub(a, b);
+    } else if constexpr (R == 3) {
+        const float s3 = 0.86602540378443864676f;
+        float2 t1 = cadd(v[1], v[2]);
+        float2 t2 = make_float2(v[0].x - 0.5f * t1.x, v[0].y - 0.5f * t1.y);
+        float2 d = csub(v[1], v[2]);
+        float2 t3 = mul_mi<INV>(make_float2(s3 * d.x, s3 * d.y));
+        v[0] = cadd(v[0], t1);
+        v[1] = cadd(t2, t3);
+        v[2] = csub(t2, t3);
+    } else if constexpr (R == 4) {
+        float2 a0 = cadd(v[0], v[2]), a1 = csub(v[0], v[2]);
+        float2 a2 = cadd(v[1], v[3]), a3 = mul_mi<INV>(csub(v[1], v[3]));
+        v[0] = cadd(a0, a2);
+        v[1] = cadd(a1, a3);
+        v[2] = csub(a0, a2);
+        v[3] = csub(a1, a3);
+    } else if constexpr (R == 5) {
+        const float c1 = 0.30901699437494742410f, c2 = -0.80901699437494742410f;
+        const float s1 = 0.95105651629515357212f, s2 = 0.58778525229247312917f;
+        float2 p1 = cadd(v[1], v[4]), m1 = csub(v[1], v[4]);
+        float2 p2 = cadd(v[2], v[3]), m2 = csub(v[2], v[3]);
+        float2 e1 = make_float2(v[0].x + c1 * p1.x + c2 * p2.x, v[0].y + c1 * p1.y + c2 * p2.y);
+        float2 e2 = make_float2(v[0].x + c2 * p1.x + c1 * p2.x, v[0].y + c2 * p1.y + c1 * p2.y);
+        float2 f1 = mul_mi<INV>(make_float2(s1 * m1.x + s2 * m2.x, s1 * m1.y + s2 * m2.y));
+        float2 f2 = mul_mi<INV>(make_float2(s2 * m1.x - s1 * m2.x, s2 * m1.y - s1 * m2.y));
+        v[0] = cadd(v[0], cadd(p1, p2));
+        v[1] = cadd(e1, f1);
+        v[2] = cadd(e2, f2);
+        v[3] = csub(e2, f2);
+        v[4] = csub(e1, f1);
+    } else {
+        // R = A*B, n = n1*B + n2, k = k1 + A*k2:
+        //   X[k1 + A k2] = sum_n2 w_B^(n2 k2) w_R^(n2 k1) sum_n1 x[n1 B + n2] w_A^(n1 k1)
+        constexpr int A = first_factor(R), B = R / A;
+        static_assert(A > 1 && A < R, "radix must factor into 2, 3, 4, 5");
+        constexpr TwTab<R> tw = make_tw<R>();
+        float2 y[R];
+#pragma unroll
+        for (int n2 = 0; n2 < B; ++n2) {
+            float2 t[A];
+#pragma unroll
+            for (int n1 = 0; n1 < A; ++n1) t[n1] = v[n1 * B + n2];
+            dft<A, INV>(t);
+#pragma unroll
+            for (int k1 = 0; k1 < A; ++k1) {
+                const int idx = (n2 * k1) % R;
+                y[k1 * B + n2] = (idx == 0) ? t[k1] : cmul_tw<INV>(t[k1], make_float2(tw.c[idx], tw.s[idx]));
+            }
+        }
+#pragma unroll
+        for (int k1 = 0; k1 < A; ++k1) {
+            float2 u[B];
+#pragma unroll
+            for (int n2 = 0; n2 < B; ++n2) u[n2] = y[k1 * B + n2];
+            dft<B, INV>(u);
+#pragma unroll
+            for (int k2 = 0; k2 < B; ++k2) v[k1 + A * k2] = u[k2];
+        }
+    }
+}
+
+constexpr int FT = 256;   // threads per workgroup
+
+template <int N, int R0, int R1, int R2>
+struct Geo {
+    static_assert(R0 * R1 * R2 == N, "factorisation");
+    static constexpr int PITCH = N + 2;          // complex elements between sequences (keeps 16 B alignment, spreads banks)
+    // position of output bin m of the decimation-in-frequency passes (= input slot of bin m for decimation in time)
+    static __device__ __forceinline__ int pos(int m) {
+        const int k0 = m % R0, t = m / R0;
+        const int k1 = t % R1, k2 = t / R1;
+        return k0 * (R1 * R2) + k1 * R2 + k2;
+    }
+};
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  All channel groups of one
+// latitude go to the same XCD, back to back, so that the 64-byte pieces they read or write
+// of one order-major row meet in that XCD's L2 as whole cache lines.
+__device__ __forceinline__ bool map_block(int nlat, int ngroups, int& lat, int& group) {
+    const int id = blockIdx.x, xcd = id & 7, q = id >> 3;
+    lat = (q / ngroups) * 8 + xcd;
+    group = q % ngroups;
+    return lat < nlat;
+}
+
+// ---- forward: decimation in frequency ---------------------------------------------------------------
+template <int N, int R0, int R1, int R2, int S>
+__device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
+    using G = Geo<N, R0, R1, R2>;
+    {
+        constexpr int NB = N / R0, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                float2* base = z + p * G::PITCH + j;
+                float2 v[R0];
+#pragma unroll
+                for (int r = 0; r < R0; ++r) v[r] = base[r * NB];
+                dft<R0, 0>(v);
+                base[0] = v[0];
+#pragma unroll
+                for (int r = 1; r < R0; ++r) base[r * NB] = cmul(v[r], tw0[(r - 1) * NB + j]);
+            }
+        }
+    }
+    __syncthreads();
+    if constexpr (R2 > 1) {
+        constexpr int NB = N / R1, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                const int k0 = j / R2, n2 = j - k0 * R2;
+                float2* base = z + p * G::PITCH + k0 * (R1 * R2) + n2;
+                float2 v[R1];
+#pragma unroll
+                for (int r = 0; r < R1; ++r) v[r] = base[r * R2];
+                dft<R1, 0>(v);
+                base[0] = v[0];
+#pragma unroll
+                for (int r = 1; r < R1; ++r) base[r * R2] = cmul(v[r], tw1[(r - 1) * R2 + n2]);
+            }
+        }
+        __syncthreads();
+    }
+    {
+        constexpr int RL = (R2 > 1) ? R2 : R1;     // last radix acts on contiguous groups
+        constexpr int NB = N / RL, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                float2* base = z + p * G::PITCH + j * RL;
+                float2 v[RL];
+#pragma unroll
+                for (int r = 0; r < RL; ++r) v[r] = base[r];
+                dft<RL, 0>(v);
+#pragma unroll
+                for (int r = 0; r < RL; ++r) base[r] = v[r];
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// ---- inverse: decimation in time -------------------------------------------------------------------------
+template <int N, int R0, int R1, int R2, int S>
+__device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
+    using G = Geo<N, R0, R1, R2>;
+    {
+        constexpr int RL = (R2 > 1) ? R2 : R1;
+        constexpr int NB = N / RL, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                float2* base = z + p * G::PITCH + j * RL;
+                float2 v[RL];
+#pragma unroll
+                for (int r = 0; r < RL; ++r) v[r] = base[r];
+                dft<RL, 1>(v);
+#pragma unroll
+                for (int r = 0; r < RL; ++r) base[r] = v[r];
+            }
+        }
+    }
+    __syncthreads();
+    if constexpr (R2 > 1) {
+        constexpr int NB = N / R1, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                const int k0 = j / R2, n2 = j - k0 * R2;
+                float2* base = z + p * G::PITCH + k0 * (R1 * R2) + n2;
+                float2 v[R1];
+                v[0] = base[0];
+#pragma unroll
+                for (int r = 1; r < R1; ++r) v[r] = cmul_tw<1>(base[r * R2], tw1[(r - 1) * R2 + n2]);
+                dft<R1, 1>(v);
+#pragma unroll
+                for (int r = 0; r < R1; ++r) base[r * R2] = v[r];
+            }
+        }
+        __syncthreads();
+    }
+    {
+        constexpr int NB = N / R0, TOT = S * NB;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / NB, j = e - p * NB;
+                float2* base = z + p * G::PITCH + j;
+                float2 v[R0];
+                v[0] = base[0];
+#pragma unroll
+                for (int r = 1; r < R0; ++r) v[r] = cmul_tw<1>(base[r * NB], tw0[(r - 1) * NB + j]);
+                dft<R0, 1>(v);
+#pragma unroll
+                for (int r = 0; r < R0; ++r) base[r * NB] = v[r];
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// grid = 8 * ceil(nlat/8) * ngroups workgroups, ngroups = ceil((ld/4) / S), see map_block
+template <int N, int R0, int R1, int R2, int S>
+__global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ x,
+                                                       float* __restrict__ xm, int64_t rows, int nlat, int mmax, int ld, int ngroups, float scale) {
+    using G = Geo<N, R0, R1, R2>;
+    __shared__ __align__(16) float2 z[S * G::PITCH];
+    const int tid = threadIdx.x;
+    int lat, group;
+    if (!map_block(nlat, ngroups, lat, group)) return;
+    const int pair0 = group * S;
+    {
+        // all global loads of the workgroup are issued before the first LDS store
+        constexpr int Q = N / 4, TOT = S * Q, IT = (TOT + FT - 1) / FT;
+        float4 a[IT], b[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int e = tid + it * FT;
+            const int p = e / Q, i4 = e - p * Q;
+            const int64_t r0 = 2 * (int64_t)(pair0 + p);
+            a[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            b[it] = a[it];
+            if (e < TOT && r0 < rows) a[it] = *reinterpret_cast<const float4*>(x + (r0 * nlat + lat) * N + 4 * i4);
+            if (e < TOT && r0 + 1 < rows) b[it] = *reinterpret_cast<const float4*>(x + ((r0 + 1) * nlat + lat) * N + 4 * i4);
+        }
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / Q, i4 = e - p * Q;
+                float4* dst = reinterpret_cast<float4*>(z + p * G::PITCH + 4 * i4);
+                dst[0] = make_float4(a[it].x, b[it].x, a[it].y, b[it].y);
+                dst[1] = make_float4(a[it].z, b[it].z, a[it].w, b[it].w);
+            }
+        }
+    }
+    __syncthreads();
+    passes_dif<N, R0, R1, R2, S>(z, tw0, tw1, tid);
+    const int npairs_ld = ld / 4;
+    const float h = 0.5f * scale;
+    for (int e = tid; e < S * mmax; e += FT) {
+        const int m = e / S, p = e - m * S;
+        if (pair0 + p >= npairs_ld) continue;
+        const float2 zp = z[p * G::PITCH + G::pos(m)];
+        const float2 zq = z[p * G::PITCH + G::pos(m == 0 ? 0 : N - m)];
+        float4 o;
+        o.x = h * (zp.x + zq.x);
+        o.y = h * (zp.y - zq.y);
+        o.z = h * (zp.y + zq.y);
+        o.w = -h * (zp.x - zq.x);
+        *reinterpret_cast<float4*>(xm + ((int64_t)m * nlat + lat) * ld + 4 * (int64_t)(pair0 + p)) = o;
+    }
+}
+
+template <int N, int R0, int R1, int R2, int S>
+__global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ xm,
+                                                        float* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups) {
+    using G = Geo<N, R0, R1, R2>;
+    static_assert(N % 2 == 0, "even length");
+    __shared__ __align__(16) float2 z[S * G::PITCH];
+    const int tid = threadIdx.x;
+    int lat, group;
+    if (!map_block(nlat, ngroups, lat, group)) return;
+    const int pair0 = group * S;
+    const int npairs_ld = ld / 4;
+    constexpr int HALF = N / 2;
+    {
+        // batches of global loads first, then the scatter into digit-reversed LDS slots
+        constexpr int TOT = S * (HALF + 1), IT = (TOT + FT - 1) / FT, BATCH = 6;
+#pragma unroll
+        for (int it0 = 0; it0 < IT; it0 += BATCH) {
+            float4 v[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int e = tid + (it0 + u) * FT;
+                const int m = e / S, p = e - m * S;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (it0 + u < IT && e < TOT && m < mmax && pair0 + p < npairs_ld)
+                    v[u] = *reinterpret_cast<const float4*>(xm + ((int64_t)m * nlat + lat) * ld + 4 * (int64_t)(pair0 + p));
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int e = tid + (it0 + u) * FT;
+                if (it0 + u < IT && e < TOT) {
+                    const int m = e / S, p = e - m * S;
+                    float4 w = v[u];
+                    if (2 * (int64_t)(pair0 + p) + 1 >= rows) w.z = w.w = 0.f;     // padding slot must not leak into its partner
+                    float2* zz = z + p * G::PITCH;
+                    if (m == 0 || m == HALF) {
+                        zz[G::pos(m)] = make_float2(w.x, w.z);                     // C2R: Im of mean and Nyquist bins dropped
+                    } else {
+                        zz[G::pos(m)] = make_float2(w.x - w.w, w.y + w.z);
+                        zz[G::pos(N - m)] = make_float2(w.x + w.w, w.z - w.y);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    passes_dit<N, R0, R1, R2, S>(z, tw0, tw1, tid);
+    {
+        constexpr int Q = N / 4, TOT = S * Q;
+#pragma unroll
+        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
+            const int e = tid + it * FT;
+            if (e < TOT) {
+                const int p = e / Q, i4 = e - p * Q;
+                const int64_t r0 = 2 * (int64_t)(pair0 + p);
+                const float4* src = reinterpret_cast<const float4*>(z + p * G::PITCH + 4 * i4);
+                const float4 u0 = src[0], u1 = src[1];
+                if (r0 < rows) *reinterpret_cast<float4*>(x + (r0 * nlat + lat) * N + 4 * i4) = make_float4(u0.x, u0.z, u1.x, u1.z);
+                if (r0 + 1 < rows) *reinterpret_cast<float4*>(x + ((r0 + 1) * nlat + lat) * N + 4 * i4) = make_float4(u0.y, u0.w, u1.y, u1.w);
+            }
+        }
+    }
+}
+
+struct FastEntry {
+    int n, r0, r1, r2;
+};
+// lengths with a specialised kernel; the last radix acts on contiguous groups, an odd one keeps LDS banks apart
+const FastEntry kFast[] = {{1440, 16, 10, 9}, {480, 10, 16, 3}, {64, 8, 8, 1}, {180, 4, 5, 9}};
+
+const FastEntry* find_fast(int n) {
+    for (const auto& e : kFast)
+        if (e.n == n) return &e;
+    return nullptr;
+}
+
+template <int N, int R0, int R1, int R2>
+int go_fast(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+    constexpr int S = (N >= 1024) ? 4 : 8;
+    const int ngroups = (ld / 4 + S - 1) / S;
+    const int64_t nblocks = (int64_t)((nlat + 7) / 8) * ngroups * 8;
+    if (nblocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)nblocks);
+    if (!inverse) {
+        float scale = (float)(kTwoPi / (double)N);
+        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups, scale);
+    } else {
+        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups);
+    }
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+}  // namespace
+
+bool fft_fast_supported(int n) { return find_fast(n) != nullptr; }
+
+int fft_fast_plan_init(FftPlan& p) {
+    const FastEntry* f = find_fast(p.n);
+    if (!f) return SFNO_OK;
+    const int N = f->n, nb = N / f->r0;
+    std::vector<float2> tw0((size_t)(f->r0 - 1) * nb), tw1((size_t)std::max(1, (f->r1 - 1) * f->r2));
+    for (int k0 = 1; k0 < f->r0; ++k0)
+        for (int j = 0; j < nb; ++j) {
+            double a = -kTwoPi * (double)(((int64_t)k0 * j) % N) / (double)N;
+            tw0[(size_t)(k0 - 1) * nb + j] = make_float2((float)std::cos(a), (float)std::sin(a));
+        }
+    tw1[0] = make_float2(1.f, 0.f);
+    for (int k1 = 1; k1 < f->r1; ++k1)
+        for (int n2 = 0; n2 < f->r2; ++n2) {
+            double a = -kTwoPi * (double)(((int64_t)f->r0 * k1 * n2) % N) / (double)N;
+            tw1[(size_t)(k1 - 1) * f->r2 + n2] = make_float2((float)std::cos(a), (float)std::sin(a));
+        }
+    if (hipMalloc(&p.d_tw0, sizeof(float2) * tw0.size()) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMalloc(&p.d_tw1, sizeof(float2) * tw1.size()) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMemcpy(p.d_tw0, tw0.data(), sizeof(float2) * tw0.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
+    if (hipMemcpy(p.d_tw1, tw1.data(), sizeof(float2) * tw1.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
+    return SFNO_OK;
+}
+
+int fft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+    switch (p.n) {
+        case 1440: return go_fast<1440, 16, 10, 9>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+        case 480: return go_fast<480, 10, 16, 3>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+        case 64: return go_fast<64, 8, 8, 1>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+        case 180: return go_fast<180, 4, 5, 9>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+    }
+    return SFNO_EUNSUPPORTED;
+}
+
+}  // namespace sfno

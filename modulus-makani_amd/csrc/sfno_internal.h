@@ -67,7 +67,13 @@ struct FftPlan {
     int npass = 0;
     int radix[24];
     float2* d_tw = nullptr;        // [n] exp(-2 pi i j / n)
+    float2* d_tw0 = nullptr;       // inter-pass twiddles of the specialised kernels (fft_fast.hip)
+    float2* d_tw1 = nullptr;
 };
+bool fft_fast_supported(int n);
+int fft_fast_plan_init(FftPlan& p);
+int fft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld,
+                    hipStream_t s);
 int fft_plan_init(FftPlan& p, int n);
 void fft_plan_free(FftPlan& p);
 // x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon

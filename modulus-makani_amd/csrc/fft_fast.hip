@@ -151,7 +151,6 @@ __device__ __forceinline__ void dft(float2 (&v)[R]) {
     }
 }
 
-constexpr int FT = 256;   // threads per workgroup
 
 template <int N, int R0, int R1, int R2>
 struct Geo {
@@ -176,7 +175,7 @@ __device__ __forceinline__ bool map_block(int nlat, int ngroups, int& lat, int& 
 }
 
 // ---- forward: decimation in frequency ---------------------------------------------------------------
-template <int N, int R0, int R1, int R2, int S>
+template <int N, int R0, int R1, int R2, int S, int FT>
 __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
     using G = Geo<N, R0, R1, R2>;
     {
@@ -240,7 +239,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
 }
 
 // ---- inverse: decimation in time -------------------------------------------------------------------------
-template <int N, int R0, int R1, int R2, int S>
+template <int N, int R0, int R1, int R2, int S, int FT>
 __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
     using G = Geo<N, R0, R1, R2>;
     {
@@ -304,7 +303,7 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
 }
 
 // grid = 8 * ceil(nlat/8) * ngroups workgroups, ngroups = ceil((ld/4) / S), see map_block
-template <int N, int R0, int R1, int R2, int S>
+template <int N, int R0, int R1, int R2, int S, int FT>
 __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ x,
                                                        float* __restrict__ xm, int64_t rows, int nlat, int mmax, int ld, int ngroups, float scale) {
     using G = Geo<N, R0, R1, R2>;
@@ -339,7 +338,7 @@ __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict_
         }
     }
     __syncthreads();
-    passes_dif<N, R0, R1, R2, S>(z, tw0, tw1, tid);
+    passes_dif<N, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
     const int npairs_ld = ld / 4;
     const float h = 0.5f * scale;
     for (int e = tid; e < S * mmax; e += FT) {
@@ -356,7 +355,7 @@ __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict_
     }
 }
 
-template <int N, int R0, int R1, int R2, int S>
+template <int N, int R0, int R1, int R2, int S, int FT>
 __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ xm,
                                                         float* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups) {
     using G = Geo<N, R0, R1, R2>;
@@ -401,7 +400,7 @@ __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict
         }
     }
     __syncthreads();
-    passes_dit<N, R0, R1, R2, S>(z, tw0, tw1, tid);
+    passes_dit<N, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
     {
         constexpr int Q = N / 4, TOT = S * Q;
 #pragma unroll
@@ -434,15 +433,16 @@ const FastEntry* find_fast(int n) {
 template <int N, int R0, int R1, int R2>
 int go_fast(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     constexpr int S = (N >= 1024) ? 4 : 8;
+    constexpr int FT = (S * N >= 4096) ? 512 : 256;     // threads per workgroup
     const int ngroups = (ld / 4 + S - 1) / S;
     const int64_t nblocks = (int64_t)((nlat + 7) / 8) * ngroups * 8;
     if (nblocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
     dim3 grid((unsigned)nblocks);
     if (!inverse) {
         float scale = (float)(kTwoPi / (double)N);
-        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups, scale);
+        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S, FT>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups, scale);
     } else {
-        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups);
+        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, FT>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups);
     }
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }

@@ -33,21 +33,23 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, analysis ? 0 : 1, p.csphase);
     std::vector<float> packed;
     std::vector<int64_t> aoff;
-    pack_legendre(gen, quad_w, analysis, packed, aoff);
+    pack_legendre_fold(gen, quad_w, analysis, packed, aoff);
+    // a workgroup covers two 32-row blocks of each parity
+    const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
     std::vector<double> cost(p.mmax);
     for (int m = 0; m < p.mmax; ++m) {
-        int nl = std::max(0, p.lmax - m);
+        int nl0 = (p.lmax - m > 0) ? (p.lmax - m + 1) / 2 : 0;
         if (analysis) {
-            nrb[m] = (nl + PG_ROWS - 1) / PG_ROWS;
+            nrb[m] = (nl0 + PG_ROWS - 1) / PG_ROWS;
             cost[m] = 1.0;
         } else {
-            nrb[m] = (p.nlat + PG_ROWS - 1) / PG_ROWS;    // orders without any degree still zero-fill their rows
-            cost[m] = 1.0 + (nl + PG_KC - 1) / PG_KC;
+            nrb[m] = (K2 + PG_ROWS - 1) / PG_ROWS;       // orders without any degree still zero-fill their rows
+            cost[m] = 1.0 + (nl0 + PG_KC - 1) / PG_KC;
         }
     }
     std::vector<int2> work;
-    build_worklist(nrb, cost, work);
+    build_worklist(nrb, cost, work, 2);
     t.n_work = (int)work.size();
     t.n_blocks = (int64_t)(packed.size() / PG_BLOCK_FLOATS);
     int rc;
@@ -176,7 +178,7 @@ extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, f
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->fwd, xm, spec, ld);
-    return pgemm_launch(PG_ANALYSIS, a, p->fwd.n_work, ld, (hipStream_t)stream);
+    return legendre_fold_launch(true, a, p->fwd.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec, float* xm, int64_t rows, void* stream) {
@@ -184,7 +186,7 @@ extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv, spec, xm, ld);
-    return pgemm_launch(PG_SYNTHESIS, a, p->inv.n_work, ld, (hipStream_t)stream);
+    return legendre_fold_launch(false, a, p->inv.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const float* x, float* spec, int64_t rows, void* workspace,

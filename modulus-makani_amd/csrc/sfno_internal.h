@@ -59,7 +59,12 @@ struct LegendreGen {
 void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
                    std::vector<int64_t>& aoff);
 // XCD-aware work list: cost[b] = relative time of one workgroup of batch b, nrb[b] = row blocks
-void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work);
+void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work,
+                    int rb_step = PG_WAVES);
+// equator-folded Legendre streams (two per order: even and odd l+m), see tables.cpp
+void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+                        std::vector<int64_t>& aoff);
+int legendre_fold_launch(bool analysis, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
 struct FftPlan {

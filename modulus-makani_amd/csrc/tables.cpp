@@ -217,7 +217,50 @@ void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, st
     });
 }
 
-void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work) {
+// Folded tables: the grids are symmetric about the equator and Pbar_l^m(pi - theta) =
+// (-1)^(l+m) Pbar_l^m(theta), so degrees of even and odd l+m only need the northern half of the
+// latitudes, applied to the sum resp. difference of mirrored rows.  Per order m and parity p
+// (l = m + p + 2 i) one packed stream:
+//   analysis : rows = i, K = latitude k < ceil(nlat/2), value P*w (the equator row counted once)
+//   synthesis: rows = latitude k < ceil(nlat/2), K = i (both parities padded to the chunk count of p = 0)
+// aoff[2*m + p] = first block of that stream.
+void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+                        std::vector<int64_t>& aoff) {
+    const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
+    const int K2 = (nlat + 1) / 2;
+    auto nl_p = [&](int m, int p) { return (lmax - m - p > 0) ? (lmax - m - p + 1) / 2 : 0; };
+    aoff.assign((size_t)2 * mmax, 0);
+    int64_t tot = 0;
+    for (int m = 0; m < mmax; ++m)
+        for (int p = 0; p < 2; ++p) {
+            aoff[2 * m + p] = tot;
+            int64_t nrb = analysis ? (nl_p(m, p) + PG_ROWS - 1) / PG_ROWS : (K2 + PG_ROWS - 1) / PG_ROWS;
+            int64_t nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl_p(m, 0) + PG_KC - 1) / PG_KC;
+            tot += nrb * nc;
+        }
+    packed.assign((size_t)tot * PG_BLOCK_FLOATS, 0.0f);
+    float* base = packed.data();
+    parallel_for(mmax, [&, base](int m) {
+        int nl = lmax - m;
+        if (nl <= 0) return;
+        std::vector<double> rows((size_t)nl * nlat);
+        g.rows_for_m(m, rows.data());
+        const double* r = rows.data();
+        for (int p = 0; p < 2; ++p) {
+            const int np = nl_p(m, p);
+            float* dst = base + (size_t)aoff[2 * m + p] * PG_BLOCK_FLOATS;
+            if (analysis) {
+                pack_blocks(dst, np, K2, [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * quad_w[k]; });
+            } else {
+                // K extent padded to the even-parity chunk count so that both parities run the same loop
+                const int kpad = nl_p(m, 0);
+                pack_blocks(dst, K2, kpad, [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] : 0.0; });
+            }
+        }
+    });
+}
+
+void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work, int rb_step) {
     // Workgroups are handed to the 8 XCDs round-robin by linear id, so entry 8*i + x of the
     // list runs on XCD x.  All workgroups of one batch share their Q panel through that XCD's
     // L2, so a batch is never split across queues; batches are assigned longest-first to the
@@ -225,7 +268,7 @@ void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost
     const int nb = (int)nrb.size();
     std::vector<int> order(nb);
     std::iota(order.begin(), order.end(), 0);
-    auto total = [&](int b) { return cost[b] * ((nrb[b] + PG_WAVES - 1) / PG_WAVES); };
+    auto total = [&](int b) { return cost[b] * ((nrb[b] + rb_step - 1) / rb_step); };
     std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return total(a) > total(b); });
     std::vector<std::vector<int2>> q(8);
     double load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -234,7 +277,7 @@ void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost
         int best = 0;
         for (int x = 1; x < 8; ++x)
             if (load[x] < load[best]) best = x;
-        for (int rb = 0; rb < nrb[b]; rb += PG_WAVES) q[best].push_back(make_int2(b, rb));
+        for (int rb = 0; rb < nrb[b]; rb += rb_step) q[best].push_back(make_int2(b, rb));
         load[best] += total(b);
     }
     size_t len = 0;

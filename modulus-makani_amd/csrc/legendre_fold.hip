@@ -16,9 +16,10 @@
 namespace sfno {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
 template <int NT, bool ANALYSIS>
-__global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
+__global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     constexpr int TN = 32 * NT;
     constexpr int LDQ = TN + ((TN % 64 == 0) ? 32 : 0);
     // [buffer][parity][k][column]; reused for the parity exchange of the synthesis epilogue
@@ -27,7 +28,8 @@ __global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
     const int2 wi = a.work[blockIdx.x];
     const int m = wi.x;
     if (m < 0) return;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int par = wave >> 1, rb = wi.y + (wave & 1);
     const int n0 = blockIdx.y * TN;
     const int ld = a.ld, nlat = a.nlat, lmax = a.lmax;
@@ -41,11 +43,11 @@ __global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
     const int nrb = (nrows + PG_ROWS - 1) / PG_ROWS;
     const int nc = ANALYSIS ? (K2 + PG_KC - 1) / PG_KC : (nl0 + PG_KC - 1) / PG_KC;
     const bool active = rb < nrb;
-    const int tiles = min(NT, (ld - n0 + 31) / 32);
 
     const float* xm_m = (ANALYSIS ? a.Q : a.Out) + (int64_t)m * nlat * ld;     // Fourier panel of order m
     const float* sp_m = (ANALYSIS ? a.Out : a.Q) + (int64_t)m * lmax * ld;     // spectral panel of order m
-    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((a.a_off[2 * m + par] + (int64_t)(active ? rb : 0) * nc) * 128 + lane);
+    // wavefronts without a row block read the head of the table (always at least nc blocks long) and discard it
+    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((active ? a.a_off[2 * m + par] + (int64_t)rb * nc : (int64_t)0) * 128 + lane);
 
     floatx16 acc[NT];
 #pragma unroll
@@ -54,86 +56,99 @@ __global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
         for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
 
     constexpr int QV = (NT + 1) / 2;       // float4 per thread per 16-row panel
-    float4 q0[QV], q1[QV];
+    f4 q0[QV], q1[QV];
 
+    // Loads are unconditional (indices clamped into the panel) and keep the raw rows in
+    // registers; masking and the mirror sum/difference happen when the chunk is written to
+    // LDS, one chunk of MFMAs later.
     auto q_load = [&](int c) {
 #pragma unroll
         for (int u = 0; u < QV; ++u) {
             const int e = tid + 256 * u;
             const int row = e / (TN / 4), c4 = e - row * (TN / 4);
-            const int i = c * PG_KC + row, n = n0 + 4 * c4;
-            float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-            if (e < 4 * TN && n < ld) {
-                if (ANALYSIS) {
-                    // i = latitude k; panel 0 = X[k] + X[k'], panel 1 = X[k] - X[k']
-                    if (i < K2) {
-                        const int kk = nlat - 1 - i;
-                        const float4 x0 = *reinterpret_cast<const float4*>(xm_m + (int64_t)i * ld + n);
-                        if (kk != i) {
-                            const float4 x1 = *reinterpret_cast<const float4*>(xm_m + (int64_t)kk * ld + n);
-                            v0 = make_float4(x0.x + x1.x, x0.y + x1.y, x0.z + x1.z, x0.w + x1.w);
-                            v1 = make_float4(x0.x - x1.x, x0.y - x1.y, x0.z - x1.z, x0.w - x1.w);
-                        } else {
-                            v0 = x0;                      // the equator row is its own mirror image
-                        }
-                    }
-                } else {
-                    // i = index within a parity; panel 0 = degree m+2i, panel 1 = degree m+2i+1
-                    const int l0 = m + 2 * i;
-                    if (l0 < lmax) v0 = *reinterpret_cast<const float4*>(sp_m + (int64_t)l0 * ld + n);
-                    if (l0 + 1 < lmax) v1 = *reinterpret_cast<const float4*>(sp_m + (int64_t)(l0 + 1) * ld + n);
-                }
+            const int i = c * PG_KC + row, n = min(n0 + 4 * c4, ld - 4);
+            if (ANALYSIS) {
+                const int k = min(i, K2 - 1);
+                q0[u] = *reinterpret_cast<const f4*>(xm_m + (int64_t)k * ld + n);
+                q1[u] = *reinterpret_cast<const f4*>(xm_m + (int64_t)(nlat - 1 - k) * ld + n);
+            } else {
+                const int l0 = min(m + 2 * i, lmax - 1), l1 = min(m + 2 * i + 1, lmax - 1);
+                q0[u] = *reinterpret_cast<const f4*>(sp_m + (int64_t)l0 * ld + n);
+                q1[u] = *reinterpret_cast<const f4*>(sp_m + (int64_t)l1 * ld + n);
             }
-            q0[u] = v0;
-            q1[u] = v1;
         }
     };
-    auto q_store = [&](int buf) {
+    auto q_store = [&](int buf, int c) {
+        const f4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int u = 0; u < QV; ++u) {
             const int e = tid + 256 * u;
             const int row = e / (TN / 4), c4 = e - row * (TN / 4);
+            const int i = c * PG_KC + row;
+            const bool col_ok = n0 + 4 * c4 < ld;
             if (e < 4 * TN) {
-                *reinterpret_cast<float4*>(&qs[buf][0][row][4 * c4]) = q0[u];
-                *reinterpret_cast<float4*>(&qs[buf][1][row][4 * c4]) = q1[u];
+                f4 v0, v1;
+                if (ANALYSIS) {
+                    // i = latitude k; panel 0 = X[k] + X[k'], panel 1 = X[k] - X[k']; the equator row is its own mirror
+                    const bool ok = col_ok && i < K2, mirror = (nlat - 1 - i) != i;
+                    v0 = mirror ? q0[u] + q1[u] : q0[u];
+                    v1 = mirror ? q0[u] - q1[u] : zero;
+                    v0 = ok ? v0 : zero;
+                    v1 = ok ? v1 : zero;
+                } else {
+                    // i = index within a parity; panel 0 = degree m+2i, panel 1 = degree m+2i+1
+                    v0 = (col_ok && m + 2 * i < lmax) ? q0[u] : zero;
+                    v1 = (col_ok && m + 2 * i + 1 < lmax) ? q1[u] : zero;
+                }
+                *reinterpret_cast<f4*>(&qs[buf][0][row][4 * c4]) = v0;
+                *reinterpret_cast<f4*>(&qs[buf][1][row][4 * c4]) = v1;
             }
         }
     };
-
-    float4 acur[2], anext[2];
-    q_load(0);
-    if (active && nc > 0) {
-        acur[0] = ap[0];
-        acur[1] = ap[64];
-    }
-    q_store(0);
-    __syncthreads();
-
     const int kh = lane >> 5, cl = lane & 31;
+    // One K-chunk of MFMAs.  No branches inside: columns past ld hold zeros in LDS and are
+    // masked at the store, so the LDS reads can be issued well ahead of the matrix instructions.
+    auto compute = [&](int buf, const f4 (&ar)[2]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float* qrow = &qs[buf][par][8 * h + 2 * s + kh][cl];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[h][s], qrow[32 * t], acc[t], 0, 0, 0);
+            }
+        }
+    };
+    const f4* apv = reinterpret_cast<const f4*>(ap);
+    auto a_load = [&](int c, f4 (&ar)[2]) {
+        ar[0] = apv[(int64_t)c * 128];
+        ar[1] = apv[(int64_t)c * 128 + 64];
+    };
+
+    // Software pipeline, one chunk deep: the loads of chunk c+1 (raw panel rows and table
+    // fragments) are issued before the MFMAs of chunk c and are first touched after them.
+    // The explicit wait for all of them at the end of the iteration keeps the wait-count
+    // bookkeeping of the next iteration's MFMA block empty.
+    f4 acur[2], anext[2];
+    if (nc > 0) {
+        q_load(0);
+        a_load(0, acur);
+        q_store(0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): the first table fragments too
+    __syncthreads();
     for (int c = 0; c < nc; ++c) {
         const int buf = c & 1;
         const bool more = c + 1 < nc;
         if (more) {
             q_load(c + 1);
-            if (active) {
-                anext[0] = ap[(int64_t)(c + 1) * 128];
-                anext[1] = ap[(int64_t)(c + 1) * 128 + 64];
-            }
+            a_load(c + 1, anext);
         }
-        if (active) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const float af[4] = {acur[h].x, acur[h].y, acur[h].z, acur[h].w};
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const float* qrow = &qs[buf][par][8 * h + 2 * s + kh][cl];
-#pragma unroll
-                    for (int t = 0; t < NT; ++t)
-                        if (t < tiles) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], qrow[32 * t], acc[t], 0, 0, 0);
-                }
-            }
-        }
-        if (more) q_store(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (active) compute(buf, acur);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) q_store(buf ^ 1, c + 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): everything issued above has landed
         __syncthreads();
         acur[0] = anext[0];
         acur[1] = anext[1];
@@ -145,7 +160,6 @@ __global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
         float* out = a.Out + (int64_t)m * lmax * ld;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            if (t >= tiles) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = PG_ROWS * rb + 8 * (v >> 2) + 4 * kh + (v & 3);
@@ -167,8 +181,7 @@ __global__ __launch_bounds__(256) void legendre_fold_kernel(PgemmArgs a) {
             float* out = a.Out + (int64_t)m * nlat * ld;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                if (t >= tiles) continue;
-#pragma unroll
+    #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int k = PG_ROWS * rb + 8 * (v >> 2) + 4 * kh + (v & 3);
                     const int n = n0 + 32 * t + cl;

@@ -258,37 +258,23 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
     if (!w) return SFNO_ENOMEM;
     w->I = I; w->O = O; w->L = L; w->compute = compute;
     if (hipGetDevice(&w->device) != hipSuccess) { delete w; return SFNO_EHIP; }
-    w->nrb = (2 * O + PG_ROWS - 1) / PG_ROWS;
+    w->nob = (2 * O + DH_COLS - 1) / DH_COLS;
     w->nc = (2 * I + PG_KC - 1) / PG_KC;
-    const int64_t per_l = (int64_t)w->nrb * w->nc;
-    w->tab.n_blocks = per_l * L;
-    std::vector<int64_t> aoff(L);
-    std::vector<int> nrb(L, w->nrb);
-    std::vector<double> cost(L);
-    for (int l = 0; l < L; ++l) {
-        aoff[l] = per_l * l;
-        cost[l] = 1.0 + l;      // a forward transform fills orders m <= l only
-    }
-    std::vector<int2> work;
-    build_worklist(nrb, cost, work);
-    w->tab.n_work = (int)work.size();
-    int rc = SFNO_OK;
-    if (hipMalloc((void**)&w->tab.d_A, sizeof(float) * (size_t)w->tab.n_blocks * PG_BLOCK_FLOATS) != hipSuccess) rc = SFNO_ENOMEM;
-    if (rc == SFNO_OK) rc = upload(&w->tab.d_aoff, aoff);
-    if (rc == SFNO_OK) rc = upload(&w->tab.d_work, work);
-    if (rc != SFNO_OK) { sfno_dhconv_weights_destroy(w); return rc; }
+    // 8 x 64 complex numbers per (degree, column block, chunk)
+    const size_t bytes = sizeof(float) * 1024 * (size_t)L * w->nob * w->nc;
+    if (hipMalloc((void**)&w->d_W, bytes) != hipSuccess) { delete w; return SFNO_ENOMEM; }
     *out = w;
     return SFNO_OK;
 }
 
 extern "C" int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream) {
     if (!w || !weight) return SFNO_EINVAL;
-    return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->tab.d_A, w->I, w->O, w->L, (hipStream_t)stream);
+    return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, (hipStream_t)stream);
 }
 
 extern "C" int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w) {
     if (!w) return SFNO_OK;
-    free_table(w->tab);
+    if (w->d_W) (void)hipFree(w->d_W);
     delete w;
     return SFNO_OK;
 }
@@ -296,13 +282,10 @@ extern "C" int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w) {
 extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* spec_in, float* spec_out, int batch, int mmax,
                                     int triangular, void* stream) {
     if (!w || !spec_in || !spec_out || batch < 1 || mmax < 1) return SFNO_EINVAL;
-    PgemmArgs a;
-    std::memset(&a, 0, sizeof(a));
-    a.A = w->tab.d_A;
-    a.a_off = w->tab.d_aoff;
-    a.work = w->tab.d_work;
-    a.Q = spec_in;
-    a.Out = spec_out;
+    DhconvArgs a;
+    a.X = spec_in;
+    a.W = w->d_W;
+    a.Y = spec_out;
     a.B = batch;
     a.I2 = 2 * w->I;
     a.O2 = 2 * w->O;
@@ -311,7 +294,9 @@ extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* s
     a.tri = triangular ? 1 : 0;
     a.ld_in = (int)sfno_spectral_ld((int64_t)batch * w->I);
     a.ld_out = (int)sfno_spectral_ld((int64_t)batch * w->O);
-    return pgemm_launch(PG_DHCONV, a, w->tab.n_work, (int64_t)mmax * batch, (hipStream_t)stream);
+    a.nob = w->nob;
+    a.nc = w->nc;
+    return dhconv_launch(a, (hipStream_t)stream);
 }
 
 extern "C" size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int mmax) {

@@ -1,8 +1,7 @@
 // Layout passes between the reference coefficient layout (complex64 [rows][lmax][mmax],
 // m fastest -- what RealSHT.forward returns and InverseRealSHT.forward / the dhconv einsum
 // consume, makani/models/common/spectral_convolution.py:131-141) and the order-major
-// "spectral" layout float [mmax][lmax][ld] the contraction kernels work on, plus the
-// packing of a SpectralConv weight into the per-degree MFMA operand stream.
+// "spectral" layout float [mmax][lmax][ld] the contraction kernels work on.
 #include "sfno_internal.h"
 
 namespace sfno {
@@ -58,36 +57,6 @@ __global__ __launch_bounds__(256) void coeffs_to_spectral_kernel(const float2* _
     }
 }
 
-// One thread per float4 of the packed stream of degree l (see sfno_internal.h for the block layout).
-// W'[2o+c][2i+d] of the real embedding of y = sum_i x_i w_io:  (c,d)=(0,0): re, (0,1): -im, (1,0): im, (1,1): re.
-__global__ __launch_bounds__(256) void dhconv_pack_kernel(const float2* __restrict__ w, float4* __restrict__ packed, int I, int O, int L,
-                                                          int nrb, int nc) {
-    const int64_t per_l = (int64_t)nrb * nc * 128;    // float4 per degree
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= per_l * L) return;
-    const int l = (int)(idx / per_l);
-    int64_t rem = idx - (int64_t)l * per_l;
-    const int j = (int)(rem & 63);
-    const int h = (int)((rem >> 6) & 1);
-    const int64_t blk = rem >> 7;
-    const int c = (int)(blk % nc), rb = (int)(blk / nc);
-    const int row = PG_ROWS * rb + (j & 31);
-    const int o = row >> 1, cc = row & 1;
-    float out[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        const int k = PG_KC * c + 8 * h + 2 * s + (j >> 5);
-        const int i = k >> 1, d = k & 1;
-        float v = 0.f;
-        if (o < O && i < I) {
-            const float2 z = w[((int64_t)i * O + o) * L + l];
-            v = (cc == d) ? z.x : (cc ? z.y : -z.y);
-        }
-        out[s] = v;
-    }
-    packed[idx] = make_float4(out[0], out[1], out[2], out[3]);
-}
-
 static bool grid_ok(int64_t rows, int lmax) { return rows > 0 && lmax > 0 && lmax <= 65535 && (rows + 31) / 32 <= 65535; }
 
 int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri, hipStream_t s) {
@@ -102,15 +71,6 @@ int spectral_to_coeffs_launch(const float* spec, float2* coeffs, int64_t rows, i
     if (!grid_ok(rows, lmax) || mmax <= 0 || ld < 2 * rows) return SFNO_EINVAL;
     dim3 grid((mmax + 31) / 32, lmax, (unsigned)((rows + 31) / 32));
     hipLaunchKernelGGL(spectral_to_coeffs_kernel, grid, dim3(32, 8), 0, s, spec, coeffs, rows, lmax, mmax, ld, tri);
-    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
-}
-
-int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, hipStream_t s) {
-    const int nrb = (2 * O + PG_ROWS - 1) / PG_ROWS, nc = (2 * I + PG_KC - 1) / PG_KC;
-    const int64_t total = (int64_t)nrb * nc * 128 * L;
-    const int64_t blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    hipLaunchKernelGGL(dhconv_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<float4*>(packed), I, O, L, nrb, nc);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

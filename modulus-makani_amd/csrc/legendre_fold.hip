@@ -109,14 +109,21 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     // One K-chunk of MFMAs.  No branches inside: columns past ld hold zeros in LDS and are
     // masked at the store, so the LDS reads can be issued well ahead of the matrix instructions.
     auto compute = [&](int buf, const f4 (&ar)[2]) {
+        // the panel values of k-step i+1 are read from LDS before the MFMAs of k-step i are issued
+        float qv[2][NT];
+        const float* qbase = &qs[buf][par][kh][cl];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int t = 0; t < NT; ++t) qv[0][t] = qbase[32 * t];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float* qrow = &qs[buf][par][8 * h + 2 * s + kh][cl];
+        for (int i = 0; i < 8; ++i) {
+            if (i + 1 < 8) {
+                const float* qrow = qbase + 2 * (i + 1) * LDQ;
 #pragma unroll
-                for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[h][s], qrow[32 * t], acc[t], 0, 0, 0);
+                for (int t = 0; t < NT; ++t) qv[(i + 1) & 1][t] = qrow[32 * t];
             }
+            const float av = ar[i >> 2][i & 3];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, qv[i & 1][t], acc[t], 0, 0, 0);
         }
     };
     const f4* apv = reinterpret_cast<const f4*>(ap);

@@ -8,20 +8,18 @@
 
 namespace sfno {
 
-// ---- packed-operand GEMM ("pgemm") ---------------------------------------------------
+// ---- packed operands -------------------------------------------------------------------
 // One operand of every contraction on this path is constant between calls (Legendre
 // table, SpectralConv weight).  It is stored as a stream of 32x16 blocks, each laid out
 // exactly as the MFMA fragments of one wavefront consume it: block = 2 halves x 64 lanes
 // x float4; lane j of half h holds, for s = 0..3,
 //     P[row = 32*rb + (j & 31)][k = 16*c + 8*h + 2*s + (j >> 5)].
-// A wavefront owns one 32-row block `rb` of one batch (order m or degree l) and walks its
-// K-chunks c = 0..nc-1, which are contiguous in memory.
+// A wavefront owns one 32-row block `rb` of one batch (order m and parity, or degree l) and
+// walks its K-chunks c = 0..nc-1, which are contiguous in memory.
 constexpr int PG_ROWS = 32;        // rows per block (MFMA 32x32x2)
 constexpr int PG_KC = 16;          // K per block
 constexpr int PG_BLOCK_FLOATS = PG_ROWS * PG_KC;   // 512 floats = 2 KiB
 constexpr int PG_WAVES = 4;        // wavefronts (= row blocks) per workgroup
-
-enum PgemmMode { PG_ANALYSIS = 0, PG_SYNTHESIS = 1, PG_DHCONV = 2 };
 
 struct PgemmTable {
     float* d_A = nullptr;          // packed stream
@@ -39,11 +37,18 @@ struct PgemmArgs {
     float* Out;
     int lmax, nlat, mmax;          // Legendre modes
     int ld;                        // channel leading dimension of Q and Out (Legendre modes)
-    // dhconv mode
-    int B, I2, O2, L, M, tri, ld_in, ld_out;
 };
 
-int pgemm_launch(int mode, const PgemmArgs& a, int n_work, int64_t ncols_max, hipStream_t s);
+// dhconv: output columns o' per workgroup, and the kernel arguments
+constexpr int DH_COLS = 128;
+struct DhconvArgs {
+    const float* X;                // spectral layout, rows (m, l, b) of 2*I floats
+    const float* W;                // packed complex weights [L][nob][nc][8][64]
+    float* Y;                      // spectral layout, rows of 2*O floats
+    int B, I2, O2, L, M, tri, ld_in, ld_out;
+    int nob, nc;                   // column blocks of DH_COLS over 2*O, K chunks of 16 over 2*I
+};
+int dhconv_launch(const DhconvArgs& a, hipStream_t s);
 
 // ---- host-side table construction (tables.cpp) -----------------------------------------
 int quadrature(int grid, int nlat, double* theta, double* w);
@@ -55,9 +60,6 @@ struct LegendreGen {
     LegendreGen(int mmax, int lmax, int nlat, const double* theta, int norm, int inverse, int csphase);
     void rows_for_m(int m, double* out) const;
 };
-// packed analysis (weights = P*w) or synthesis (P) streams, and the per-batch block offsets
-void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
-                   std::vector<int64_t>& aoff);
 // XCD-aware work list: cost[b] = relative time of one workgroup of batch b, nrb[b] = row blocks
 void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work,
                     int rb_step = PG_WAVES);
@@ -103,6 +105,6 @@ struct sfno_sht_plan {
 
 struct sfno_dhconv_weights {
     int I, O, L, compute, device;
-    int nrb, nc;                   // row blocks (over 2*O) and K chunks (over 2*I) per degree
-    sfno::PgemmTable tab;
+    int nob, nc;                   // column blocks (over 2*O) and K chunks (over 2*I) per degree
+    float* d_W = nullptr;          // packed complex weights
 };

@@ -186,37 +186,6 @@ static void pack_blocks(float* dst, int rows, int K, G get) {
         }
 }
 
-void pack_legendre(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
-                   std::vector<int64_t>& aoff) {
-    const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
-    aoff.assign(mmax, 0);
-    int64_t tot = 0;
-    for (int m = 0; m < mmax; ++m) {
-        aoff[m] = tot;
-        int nl = std::max(0, lmax - m);
-        int64_t nrb = analysis ? (nl + PG_ROWS - 1) / PG_ROWS : (nlat + PG_ROWS - 1) / PG_ROWS;
-        int64_t nc = analysis ? (nlat + PG_KC - 1) / PG_KC : (nl + PG_KC - 1) / PG_KC;
-        tot += nrb * nc;
-    }
-    packed.assign((size_t)tot * PG_BLOCK_FLOATS, 0.0f);
-    float* base = packed.data();
-    parallel_for(mmax, [&, base](int m) {
-        int nl = lmax - m;
-        if (nl <= 0) return;
-        std::vector<double> rows((size_t)nl * nlat);
-        g.rows_for_m(m, rows.data());
-        float* dst = base + (size_t)aoff[m] * PG_BLOCK_FLOATS;
-        const double* r = rows.data();
-        if (analysis) {
-            // rows = l - m, K = latitude; value = P * w_k
-            pack_blocks(dst, nl, nlat, [=](int row, int k) { return r[(size_t)row * nlat + k] * quad_w[k]; });
-        } else {
-            // rows = latitude, K = l - m
-            pack_blocks(dst, nlat, nl, [=](int row, int k) { return r[(size_t)k * nlat + row]; });
-        }
-    });
-}
-
 // Folded tables: the grids are symmetric about the equator and Pbar_l^m(pi - theta) =
 // (-1)^(l+m) Pbar_l^m(theta), so degrees of even and odd l+m only need the northern half of the
 // latitudes, applied to the sum resp. difference of mirrored rows.  Per order m and parity p

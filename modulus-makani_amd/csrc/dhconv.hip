@@ -35,7 +35,10 @@ __global__ __launch_bounds__(256) void dhconv_kernel(DhconvArgs a) {
     const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
     if (lidx >= a.L) return;
     const int l = a.L - 1 - lidx;
-    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    // Wavefront w of every workgroup runs on SIMD w, and low degrees fill only the first row blocks:
+    // rotate the block a wavefront takes from workgroup to workgroup so that no SIMD gets all the work.
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
     const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;      // rows (m,b) present at this degree
     const int r0 = blockIdx.y * 128;
     if (r0 >= ncols) return;

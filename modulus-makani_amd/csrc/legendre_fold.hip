@@ -30,7 +30,10 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     if (m < 0) return;
     // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const int par = wave >> 1, rb = wi.y + (wave & 1);
+    // wavefront w runs on SIMD w; alternate which SIMDs get the (possibly absent) second row block
+    // and the (one row shorter) odd parity from workgroup to workgroup
+    const int wslot = (wave + blockIdx.x) & 3;
+    const int par = wslot >> 1, rb = wi.y + (wslot & 1);
     const int n0 = blockIdx.y * TN;
     const int ld = a.ld, nlat = a.nlat, lmax = a.lmax;
     if (n0 >= ld) return;
@@ -176,7 +179,7 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
         }
     } else {
         // odd-parity wavefronts hand their sums to the even-parity wavefront of the same row block
-        float* exch = &qs[0][0][0][0] + (wave & 1) * (NT * 16 * 64);
+        float* exch = &qs[0][0][0][0] + (wslot & 1) * (NT * 16 * 64);
         if (par == 1 && active) {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -208,7 +211,8 @@ template <bool ANALYSIS>
 static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     const int64_t ncols = a.ld;
     if (n_work <= 0 || ncols <= 0) return SFNO_OK;
-    static const int cand[] = {6, 5, 4, 3, 2, 1};
+    // 4 tiles keep four wavefronts per SIMD resident, 5 three; prefer the least padding, then occupancy
+    static const int cand[] = {4, 5, 3, 2, 1};
     int best = 1;
     int64_t best_pad = INT64_MAX;
     for (int nt : cand) {
@@ -222,7 +226,7 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
         break;                                                                                       \
     }
     switch (best) {
-        LF_CASE(1) LF_CASE(2) LF_CASE(3) LF_CASE(4) LF_CASE(5) LF_CASE(6)
+        LF_CASE(1) LF_CASE(2) LF_CASE(3) LF_CASE(4) LF_CASE(5)
         default: return SFNO_EINVAL;
     }
 #undef LF_CASE

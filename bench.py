@@ -32,7 +32,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block"])
+    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout"])
+    ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-channels", type=int, default=4)
     return ap.parse_args()
@@ -257,6 +258,87 @@ def bench_spectral_block(args):
     }
 
 
+def build_sfno8l(dev):
+    """SFNO-linear, 8 layers, embed 384, scale factor 3, 73 channels in/out (config/sfnonet.yaml:24-40,149-174), random init."""
+    import torch
+    from makani_amd.sfnonet import SphericalFourierNeuralOperatorNet
+
+    torch.manual_seed(4)
+    net = SphericalFourierNeuralOperatorNet(inp_shape=(721, 1440), out_shape=(721, 1440), scale_factor=3, inp_chans=73, out_chans=73,
+                                            embed_dim=384, num_layers=8, use_mlp=True, mlp_ratio=2.0, activation_function="gelu",
+                                            normalization_layer="instance_norm", big_skip=True, operator_type="dhconv", filter_type="linear")
+    return net.to(dev).eval()
+
+
+def time_sfno_forward(batch, iters, warmup, dev):
+    """Median forward time (ms) of the SFNO-8L under bf16 autocast, inference mode, HIP events."""
+    import torch
+
+    net = build_sfno8l(dev)
+    x = torch.randn(batch, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
+    times = []
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        for _ in range(warmup):
+            y = net(x)
+        torch.cuda.synchronize()
+        for _ in range(iters):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            y = net(x)
+            e.record()
+            torch.cuda.synchronize()
+            times.append(s.elapsed_time(e))
+    assert torch.isfinite(y.float()).all()
+    times.sort()
+    return times[len(times) // 2], times[0], net, x
+
+
+def bench_sfno8l(args):
+    import torch
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    med, best, _, _ = time_sfno_forward(1, max(args.steps, 5), args.warmup, dev)
+    return {
+        "metric": "SFNO-L8 fwd ms/sample", "value": med, "unit": "ms/sample", "n_gpus": 1, "steps": max(args.steps, 5), "warmup": args.warmup,
+        "ms_per_step": med, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 pointwise / f32 spectral",
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: SFNO-linear 8 layers, embed 384, scale factor 3 (721x1440 -> 240x480), 73 channels, batch 1, "
+                               "bf16 autocast forward, random-init weights, N(0,1) inputs"},
+        "best_ms": best,
+    }
+
+
+def bench_rollout(args):
+    """configs[4]: batch 4, 12 autoregressive steps x_{t+1} = model(x_t) (makani/utils/inferencer.py:144-177, n_history = 0)."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    net = build_sfno8l(dev)
+    x0 = torch.randn(4, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
+    nsteps = 12
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        x = x0
+        for _ in range(2):
+            x = net(x).float()
+        torch.cuda.synchronize()
+        x = x0
+        t0 = time.perf_counter()
+        for _ in range(nsteps):
+            x = net(x).float()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    finite = bool(torch.isfinite(x).all())
+    return {
+        "metric": "SFNO-L8 rollout ms/step", "value": dt / nsteps * 1e3, "unit": "ms/step", "n_gpus": 1, "steps": nsteps, "warmup": 2,
+        "ms_per_step": dt / nsteps * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 pointwise / f32 spectral", "data": "synthetic",
+        "config": {"workload": "configs[4]: SFNO-8L, batch 4, 12-step autoregressive rollout, bf16 autocast"},
+        "ms_per_sample_step": dt / nsteps / 4 * 1e3, "finite": finite,
+    }
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -267,7 +349,20 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(1)
-    res = bench_sht_pair(args) if args.workload == "sht_pair" else bench_spectral_block(args)
+    if args.workload == "sht_pair":
+        res = bench_sht_pair(args)
+        if not args.no_sfno:
+            # the second headline figure of the metric, measured in the same run
+            torch.cuda.empty_cache()
+            med, best, _, _ = time_sfno_forward(1, 10, 3, torch.device("cuda:0"))
+            res["sfno_l8_fwd_ms_per_sample"] = {"value": med, "best": best, "batch": 1, "dtype": "bf16 pointwise / f32 spectral",
+                                                "config": "configs[3]: SFNO-linear 8 layers, embed 384, 721x1440, 73 channels, bf16 autocast"}
+    elif args.workload == "spectral_block":
+        res = bench_spectral_block(args)
+    elif args.workload == "sfno8l":
+        res = bench_sfno8l(args)
+    else:
+        res = bench_rollout(args)
     print(json.dumps(res), flush=True)
 
 

@@ -1,0 +1,254 @@
+"""Spherical Fourier Neural Operator network on the HIP spectral path.
+
+Caller-side mirror of makani/models/networks/sfnonet.py for the single-GPU, linear-filter
+configuration that Makani's recipes use (config/sfnonet.yaml:24-40,149-174): same
+constructor keywords, same layer order and parameter names (``encoder.fwd.N``,
+``blocks.i.{norm0,norm1,filter.filter,mlp.fwd.N,outer_skip}``, ``decoder.fwd.N``,
+``residual_transform``), so a Makani state_dict loads with ``strict=True``.  The spectral
+filter runs on makani_amd.SpectralConv (HIP kernels); the pointwise parts are plain
+PyTorch modules, as in the reference.
+"""
+import math
+from functools import partial
+
+import torch
+import torch.nn as nn
+
+from .sht import RealSHT, InverseRealSHT
+from .spectral_convolution import SpectralConv
+
+_ACTIVATIONS = {"relu": nn.ReLU, "gelu": nn.GELU, "silu": nn.SiLU}
+
+
+def _pointwise(cin, cout, bias, std):
+    conv = nn.Conv2d(cin, cout, 1, bias=bias)
+    nn.init.normal_(conv.weight, mean=0.0, std=std)
+    if bias:
+        nn.init.constant_(conv.bias, 0.0)
+    return conv
+
+
+class EncoderDecoder(nn.Module):
+    """Stack of 1x1 convolutions: (conv + bias, activation) x num_layers, then a bias-free conv (layers.py:86-133)."""
+
+    def __init__(self, num_layers, input_dim, output_dim, hidden_dim, act_layer, gain=1.0, input_format="nchw"):
+        super().__init__()
+        if input_format != "nchw":
+            raise NotImplementedError(f"Error, input format {input_format} not supported.")
+        mods, cur = [], input_dim
+        for _ in range(num_layers):
+            mods += [_pointwise(cur, hidden_dim, True, math.sqrt(2.0 / cur)), act_layer()]
+            cur = hidden_dim
+        mods.append(_pointwise(cur, output_dim, False, math.sqrt(gain / cur)))
+        self.fwd = nn.Sequential(*mods)
+
+    def forward(self, x):
+        return self.fwd(x)
+
+
+class MLP(nn.Module):
+    """conv1x1 -> activation -> dropout -> conv1x1 -> dropout (layers.py:136-216); parameters at fwd.0 and fwd.3."""
+
+    def __init__(self, in_features, hidden_features=None, out_features=None, act_layer=nn.GELU, output_bias=True, drop_rate=0.0,
+                 drop_type="iid", gain=1.0, **kwargs):
+        super().__init__()
+        out_features = out_features or in_features
+        hidden_features = hidden_features or in_features
+        fc1 = _pointwise(in_features, hidden_features, True, math.sqrt(2.0 / in_features))
+        fc2 = _pointwise(hidden_features, out_features, output_bias, math.sqrt(gain / hidden_features))
+        if drop_rate > 0.0:
+            drop = nn.Dropout(drop_rate) if drop_type == "iid" else nn.Dropout2d(drop_rate)
+        else:
+            drop = nn.Identity()
+        self.fwd = nn.Sequential(fc1, act_layer(), drop, fc2, drop)
+
+    def forward(self, x):
+        return self.fwd(x)
+
+
+class SpectralFilterLayer(nn.Module):
+    """Holder of the spectral operator under the name ``filter`` (sfnonet.py:51-116); linear, unfactorized filters only."""
+
+    def __init__(self, forward_transform, inverse_transform, embed_dim, filter_type="linear", operator_type="diagonal", hidden_size_factor=1,
+                 factorization=None, rank=1.0, separable=False, complex_activation="real", spectral_layers=1, bias=False, drop_rate=0.0, gain=1.0):
+        super().__init__()
+        if filter_type != "linear" or factorization is not None:
+            raise NotImplementedError("the HIP path implements filter_type='linear' without factorization")
+        self.filter = SpectralConv(forward_transform, inverse_transform, embed_dim, embed_dim, operator_type=operator_type, separable=separable,
+                                   bias=bias, gain=gain)
+
+    def forward(self, x):
+        return self.filter(x)
+
+
+class FourierNeuralOperatorBlock(nn.Module):
+    """filter -> norm0 -> (+ inner skip) -> act -> MLP -> norm1 -> (+ outer skip) (sfnonet.py:119-267)."""
+
+    def __init__(self, forward_transform, inverse_transform, embed_dim, filter_type="linear", operator_type="diagonal", mlp_ratio=2.0,
+                 mlp_drop_rate=0.0, path_drop_rate=0.0, act_layer=nn.GELU, norm_layer=(nn.Identity, nn.Identity), rank=1.0, factorization=None,
+                 separable=False, inner_skip="linear", outer_skip=None, use_mlp=False, complex_activation="real", spectral_layers=1, bias=False,
+                 final_activation=False, **kwargs):
+        super().__init__()
+        if path_drop_rate > 0.0:
+            raise NotImplementedError("stochastic depth is a training feature outside this path")
+        self.input_shape_loc = (forward_transform.nlat, forward_transform.nlon)
+        self.output_shape_loc = (inverse_transform.nlat, inverse_transform.nlon)
+        self.norm0 = norm_layer[0]()
+
+        gain_factor = 1.0 if act_layer == nn.Identity else 2.0
+        if inner_skip == "linear":
+            gain_factor /= 2.0
+            self.inner_skip = _pointwise(embed_dim, embed_dim, False, math.sqrt(gain_factor / embed_dim))
+        elif inner_skip == "identity":
+            self.inner_skip = nn.Identity()
+            gain_factor /= 2.0
+        elif inner_skip != "none":
+            raise ValueError(f"Unknown skip connection type {inner_skip}")
+
+        self.filter = SpectralFilterLayer(forward_transform, inverse_transform, embed_dim, filter_type, operator_type, hidden_size_factor=mlp_ratio,
+                                          factorization=factorization, rank=rank, separable=separable, complex_activation=complex_activation,
+                                          spectral_layers=spectral_layers, bias=bias, drop_rate=path_drop_rate, gain=gain_factor)
+        self.act_layer0 = act_layer()
+        self.norm1 = norm_layer[1]()
+
+        gain_factor = 2.0 if (final_activation and act_layer != nn.Identity) else 1.0
+        if outer_skip == "linear":
+            gain_factor /= 2.0
+            self.outer_skip = _pointwise(embed_dim, embed_dim, False, math.sqrt(gain_factor / embed_dim))
+        elif outer_skip == "identity":
+            self.outer_skip = nn.Identity()
+            gain_factor /= 2.0
+        elif outer_skip not in ("none", None):
+            raise ValueError(f"Unknown skip connection type {outer_skip}")
+
+        if use_mlp:
+            self.mlp = MLP(in_features=embed_dim, hidden_features=int(embed_dim * mlp_ratio), act_layer=act_layer, drop_rate=mlp_drop_rate,
+                           drop_type="features", gain=gain_factor)
+        if final_activation:
+            self.act_layer1 = act_layer()
+
+    def forward(self, x):
+        x, residual = self.filter(x)
+        x = self.norm0(x)
+        if hasattr(self, "inner_skip"):
+            x = x + self.inner_skip(residual)
+        x = self.act_layer0(x)
+        if hasattr(self, "mlp"):
+            x = self.mlp(x)
+        x = self.norm1(x)
+        if hasattr(self, "outer_skip"):
+            x = x + self.outer_skip(residual)
+        if hasattr(self, "act_layer1"):
+            x = self.act_layer1(x)
+        return x
+
+
+class SphericalFourierNeuralOperatorNet(nn.Module):
+    """SFNO (sfnonet.py:270-640): encoder -> num_layers blocks -> decoder, plus the big skip connection."""
+
+    def __init__(self, spectral_transform="sht", model_grid_type="equiangular", sht_grid_type="legendre-gauss", filter_type="linear",
+                 operator_type="dhconv", inp_shape=(721, 1440), out_shape=(721, 1440), scale_factor=8, inp_chans=2, out_chans=2, embed_dim=32,
+                 num_layers=4, repeat_layers=1, use_mlp=True, mlp_ratio=2.0, encoder_ratio=1, decoder_ratio=1, activation_function="gelu",
+                 encoder_layers=1, pos_embed="none", pos_drop_rate=0.0, path_drop_rate=0.0, mlp_drop_rate=0.0,
+                 normalization_layer="instance_norm", max_modes=None, hard_thresholding_fraction=1.0, big_skip=True, rank=1.0,
+                 factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0, **kwargs):
+        super().__init__()
+        if spectral_transform != "sht":
+            raise NotImplementedError("only spectral_transform='sht' runs on the HIP path")
+        self.inp_shape, self.out_shape = tuple(inp_shape), tuple(out_shape)
+        self.inp_chans, self.out_chans, self.embed_dim = inp_chans, out_chans, embed_dim
+        self.repeat_layers, self.big_skip = repeat_layers, big_skip
+        self.h = int(self.inp_shape[0] // scale_factor)
+        self.w = int(self.inp_shape[1] // scale_factor)
+        self._init_spectral_transforms(model_grid_type, sht_grid_type, hard_thresholding_fraction, max_modes)
+
+        if activation_function not in _ACTIVATIONS:
+            raise ValueError(f"Unknown activation function {activation_function}")
+        act = _ACTIVATIONS[activation_function]
+
+        self.encoder = EncoderDecoder(encoder_layers, inp_chans, embed_dim, int(encoder_ratio * embed_dim), act)
+        self.pos_drop = nn.Dropout(p=pos_drop_rate) if pos_drop_rate > 0.0 else nn.Identity()
+
+        if normalization_layer == "layer_norm":
+            raise NotImplementedError("layer_norm over channels of an nchw tensor is Makani's own distributed module; use instance_norm or none")
+        elif normalization_layer == "instance_norm":
+            norm = partial(nn.InstanceNorm2d, num_features=embed_dim, eps=1e-6, affine=True, track_running_stats=False)
+        elif normalization_layer == "none":
+            norm = nn.Identity
+        else:
+            raise NotImplementedError(f"Error, normalization {normalization_layer} not implemented.")
+
+        self.blocks = nn.ModuleList()
+        for i in range(num_layers):
+            fwd = self.trans_down if i == 0 else self.trans
+            inv = self.itrans_up if i == num_layers - 1 else self.itrans
+            self.blocks.append(
+                FourierNeuralOperatorBlock(fwd, inv, embed_dim, filter_type=filter_type, operator_type=operator_type, mlp_ratio=mlp_ratio,
+                                           mlp_drop_rate=mlp_drop_rate, path_drop_rate=0.0 if path_drop_rate == 0.0 else path_drop_rate * i / max(num_layers - 1, 1),
+                                           act_layer=act, norm_layer=(norm, norm), inner_skip="none", outer_skip="linear", use_mlp=use_mlp, rank=rank,
+                                           factorization=factorization, separable=separable, complex_activation=complex_activation,
+                                           spectral_layers=spectral_layers, bias=bias))
+
+        self.decoder = EncoderDecoder(encoder_layers, embed_dim, out_chans, int(decoder_ratio * embed_dim), act, gain=0.5 if big_skip else 1.0)
+        if big_skip:
+            self.residual_transform = _pointwise(inp_chans, out_chans, False, math.sqrt(0.5 / inp_chans))
+
+        if pos_embed == "direct":
+            self.pos_embed = nn.Parameter(torch.zeros(1, embed_dim, self.inp_shape[0], self.inp_shape[1]))
+            self.pos_embed.type = "direct"
+            with torch.no_grad():
+                nn.init.trunc_normal_(self.pos_embed, std=0.02)
+        elif pos_embed == "frequency":
+            lmax, mmax = self.itrans_up.lmax, self.itrans_up.mmax
+            rcoeffs = nn.Parameter(torch.tril(torch.randn(1, embed_dim, lmax, mmax), diagonal=0))
+            ccoeffs = nn.Parameter(torch.tril(torch.randn(1, embed_dim, lmax, mmax - 1), diagonal=-1))
+            with torch.no_grad():
+                nn.init.trunc_normal_(rcoeffs, std=0.02)
+                nn.init.trunc_normal_(ccoeffs, std=0.02)
+            self.pos_embed = nn.ParameterList([rcoeffs, ccoeffs])
+            self.pos_embed.type = "frequency"
+        elif pos_embed not in ("none", "None", None):
+            raise ValueError("Unknown position embedding type")
+
+    def _init_spectral_transforms(self, model_grid_type, sht_grid_type, hard_thresholding_fraction, max_modes):
+        # mode counts and the four transform objects exactly as sfnonet.py:503-571 derives them
+        if max_modes is not None:
+            modes_lat, modes_lon = max_modes
+        else:
+            modes_lat = int(self.h * hard_thresholding_fraction)
+            modes_lon = int((self.w // 2 + 1) * hard_thresholding_fraction)
+        self.trans_down = RealSHT(*self.inp_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type).float()
+        self.itrans_up = InverseRealSHT(*self.out_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type).float()
+        self.trans = RealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type).float()
+        self.itrans = InverseRealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type).float()
+        self.inp_shape_loc = (self.trans_down.nlat, self.trans_down.nlon)
+        self.out_shape_loc = (self.itrans_up.nlat, self.itrans_up.nlon)
+        self.h_loc, self.w_loc = self.itrans.nlat, self.itrans.nlon
+
+    def _forward_features(self, x):
+        for _ in range(self.repeat_layers):
+            for blk in self.blocks:
+                x = blk(x)
+        return x
+
+    def forward(self, x):
+        if self.big_skip:
+            if self.out_shape != self.inp_shape:
+                xtype = x.dtype
+                residual = self.itrans_up(self.trans_down(x.to(torch.float32)).contiguous()).to(dtype=xtype)
+            else:
+                residual = x
+        x = self.encoder(x)
+        if hasattr(self, "pos_embed"):
+            if self.pos_embed.type == "frequency":
+                pe = torch.stack([self.pos_embed[0], nn.functional.pad(self.pos_embed[1], (1, 0), "constant", 0)], dim=-1)
+                pe = self.itrans_up(torch.view_as_complex(pe.float().contiguous()))
+            else:
+                pe = self.pos_embed
+            x = x + pe
+        x = self.pos_drop(x)
+        x = self._forward_features(x)
+        x = self.decoder(x)
+        if self.big_skip:
+            x = x + self.residual_transform(residual)
+        return x

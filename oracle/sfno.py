@@ -1,0 +1,65 @@
+"""Float64 CPU restatement of the SFNO forward pass (oracle).
+
+Functional form of makani/models/networks/sfnonet.py:587-640 (network forward),
+119-267 (block), makani/models/common/layers.py:86-133,136-216 (1x1-conv stacks) and
+makani/models/common/spectral_convolution.py:124-148 for the linear/dhconv/instance-norm
+recipe of config/sfnonet.yaml:24-40, driven by a state_dict with Makani's key names.
+The spectral parts run on the numpy oracle, the pointwise parts on torch float64.
+"""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from .sht import ShtTables, sht_forward, sht_inverse
+from .dhconv import spectral_conv
+
+
+class SfnoOracle:
+    def __init__(self, inp_shape, out_shape, scale_factor, num_layers, model_grid_type="equiangular", sht_grid_type="legendre-gauss",
+                 activation="gelu", normalization="instance_norm", big_skip=True, use_mlp=True, hard_thresholding_fraction=1.0):
+        h, w = inp_shape[0] // scale_factor, inp_shape[1] // scale_factor
+        ml, mm = int(h * hard_thresholding_fraction), int((w // 2 + 1) * hard_thresholding_fraction)
+        self.down = ShtTables(inp_shape[0], inp_shape[1], ml, mm, model_grid_type)
+        self.up = ShtTables(out_shape[0], out_shape[1], ml, mm, model_grid_type)
+        self.mid = ShtTables(h, w, ml, mm, sht_grid_type)
+        self.inp_shape, self.out_shape = tuple(inp_shape), tuple(out_shape)
+        self.num_layers, self.big_skip, self.use_mlp = num_layers, big_skip, use_mlp
+        self.act = {"gelu": F.gelu, "relu": F.relu, "silu": F.silu}[activation]
+        self.normalization = normalization
+
+    @staticmethod
+    def _conv(x, sd, name):
+        w = sd[name + ".weight"].double()
+        b = sd.get(name + ".bias")
+        return F.conv2d(x, w, None if b is None else b.double())
+
+    def _norm(self, x, sd, name):
+        if self.normalization == "none":
+            return x
+        return F.instance_norm(x, weight=sd[name + ".weight"].double(), bias=sd[name + ".bias"].double(), eps=1e-6)
+
+    def forward(self, sd, x):
+        sd = {k: v.detach().cpu() for k, v in sd.items()}
+        x = x.detach().cpu().double()
+        if self.big_skip:
+            if self.out_shape != self.inp_shape:
+                residual = torch.from_numpy(sht_inverse(sht_forward(x.numpy(), self.down), self.up))
+            else:
+                residual = x
+        y = self._conv(self.act(self._conv(x, sd, "encoder.fwd.0")), sd, "encoder.fwd.2")
+        for i in range(self.num_layers):
+            fwd = self.down if i == 0 else self.mid
+            inv = self.up if i == self.num_layers - 1 else self.mid
+            p = f"blocks.{i}."
+            w = sd[p + "filter.filter.weight"].numpy().astype(np.complex128)
+            z, res = spectral_conv(y.numpy(), w, fwd, inv)
+            z, res = torch.from_numpy(z), torch.from_numpy(np.asarray(res))
+            z = self.act(self._norm(z, sd, p + "norm0"))
+            if self.use_mlp:
+                z = self._conv(self.act(self._conv(z, sd, p + "mlp.fwd.0")), sd, p + "mlp.fwd.3")
+            z = self._norm(z, sd, p + "norm1")
+            y = z + self._conv(res, sd, p + "outer_skip")
+        y = self._conv(self.act(self._conv(y, sd, "decoder.fwd.0")), sd, "decoder.fwd.2")
+        if self.big_skip:
+            y = y + self._conv(residual, sd, "residual_transform")
+        return y

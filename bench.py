@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="also run one plain 256 MiB elementwise copy (mul by 1): the known-size reference for FETCH_SIZE/WRITE_SIZE runs")
     ap.add_argument("--cpu-sample-channels", type=int, default=4)
     return ap.parse_args()
 
@@ -136,6 +138,10 @@ def bench_sht_pair(args):
     def step():
         return isht(sht(x))
 
+    if args.yardstick:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.mul(src, 1.0)            # reads 256 MiB, writes 256 MiB
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

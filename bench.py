@@ -164,12 +164,12 @@ def bench_sht_pair(args):
     out = torch.empty_like(x)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     stages = {
-        "rfft": lambda: check(lib.sfno_rfft(pf, P(x), P(xm), rows, sp), "rfft"),
+        "rfft": lambda: check(lib.sfno_rfft(pf, P(x), 0, P(xm), rows, sp), "rfft"),
         "legendre_analysis": lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), rows, sp), "legendre_analysis"),
         "spectral_to_coeffs": lambda: check(lib.sfno_spectral_to_coeffs(P(spec), P(coeffs), rows, lmax, mmax, 1, sp), "to_coeffs"),
         "coeffs_to_spectral": lambda: check(lib.sfno_coeffs_to_spectral(P(coeffs), P(spec), rows, lmax, mmax, 1, sp), "to_spectral"),
         "legendre_synthesis": lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), rows, sp), "legendre_synthesis"),
-        "irfft": lambda: check(lib.sfno_irfft(pi, P(xm), P(out), rows, sp), "irfft"),
+        "irfft": lambda: check(lib.sfno_irfft(pi, P(xm), P(out), 0, rows, sp), "irfft"),
     }
     stage_ms = {}
     for name, fn in stages.items():      # run in pipeline order so every buffer holds real data

@@ -58,6 +58,10 @@ extern "C" {
 #define SFNO_DIR_FORWARD 1
 #define SFNO_DIR_INVERSE 2
 
+/* element type of a grid-side (real field) tensor */
+#define SFNO_DTYPE_F32 0
+#define SFNO_DTYPE_BF16 1
+
 /* arithmetic of the Legendre / channel-mix contractions */
 #define SFNO_COMPUTE_FP32 0      /* fp32 MFMA, fp32 tables */
 #define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs, fp32 accumulate */
@@ -107,18 +111,24 @@ int sfno_sht_forward(const sfno_sht_plan* plan, const float* x, void* coeffs, in
 int sfno_sht_inverse(const sfno_sht_plan* plan, const void* coeffs, float* x, int64_t rows,
                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* Same transforms with coefficients kept in the spectral layout (no layout pass). */
-int sfno_sht_analysis(const sfno_sht_plan* plan, const float* x, float* spec, int64_t rows,
+/* Same transforms with coefficients kept in the spectral layout (no layout pass).  The grid-side
+ * tensor x may be float32 or bfloat16 (`x_dtype`, SFNO_DTYPE_*): a bf16 field is widened on load /
+ * rounded to nearest even on store inside the FFT kernels, which is what the reference's
+ * `x.float()` before and `x.to(dtype)` after the transforms compute
+ * (makani/models/common/spectral_convolution.py:127,146).  sfno_sht_io_dtype_supported tells
+ * whether the plan's longitude length has such kernels (otherwise SFNO_EUNSUPPORTED). */
+int sfno_sht_io_dtype_supported(const sfno_sht_plan* plan, int x_dtype);
+int sfno_sht_analysis(const sfno_sht_plan* plan, const void* x, int x_dtype, float* spec, int64_t rows,
                       void* workspace, size_t workspace_bytes, void* stream);
-int sfno_sht_synthesis(const sfno_sht_plan* plan, const float* spec, float* x, int64_t rows,
+int sfno_sht_synthesis(const sfno_sht_plan* plan, const float* spec, void* x, int x_dtype, int64_t rows,
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* The four stages of the transform pair on their own (what sfno_sht_analysis and
  * sfno_sht_synthesis chain).  xm is the order-major Fourier buffer float32
  * [mmax][nlat][ld]: (re,im) of 2 pi/nlon * sum_n x[r][k][n] e^{-i m phi_n} at
  * xm[m][k][2r], xm[m][k][2r+1]. */
-int sfno_rfft(const sfno_sht_plan* plan, const float* x, float* xm, int64_t rows, void* stream);
-int sfno_irfft(const sfno_sht_plan* plan, const float* xm, float* x, int64_t rows, void* stream);
+int sfno_rfft(const sfno_sht_plan* plan, const void* x, int x_dtype, float* xm, int64_t rows, void* stream);
+int sfno_irfft(const sfno_sht_plan* plan, const float* xm, void* x, int x_dtype, int64_t rows, void* stream);
 int sfno_legendre_analysis(const sfno_sht_plan* plan, const float* xm, float* spec, int64_t rows,
                            void* stream);
 int sfno_legendre_synthesis(const sfno_sht_plan* plan, const float* spec, float* xm, int64_t rows,

@@ -163,14 +163,20 @@ extern "C" int64_t sfno_fourier_elems(const sfno_sht_plan* p, int64_t rows) {
     return (int64_t)p->mmax * p->nlat * sfno_spectral_ld(rows);
 }
 
-extern "C" int sfno_rfft(const sfno_sht_plan* p, const float* x, float* xm, int64_t rows, void* stream) {
-    if (!p || !x || !xm || !rows_ok(rows)) return SFNO_EINVAL;
-    return rfft_launch(p->fft, x, xm, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+extern "C" int sfno_sht_io_dtype_supported(const sfno_sht_plan* p, int x_dtype) {
+    if (!p) return 0;
+    if (x_dtype == SFNO_DTYPE_F32) return 1;
+    return x_dtype == SFNO_DTYPE_BF16 && fft_fast_supported(p->nlon) ? 1 : 0;
 }
 
-extern "C" int sfno_irfft(const sfno_sht_plan* p, const float* xm, float* x, int64_t rows, void* stream) {
+extern "C" int sfno_rfft(const sfno_sht_plan* p, const void* x, int x_dtype, float* xm, int64_t rows, void* stream) {
     if (!p || !x || !xm || !rows_ok(rows)) return SFNO_EINVAL;
-    return irfft_launch(p->fft, xm, x, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+    return rfft_launch(p->fft, x, x_dtype, xm, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+}
+
+extern "C" int sfno_irfft(const sfno_sht_plan* p, const float* xm, void* x, int x_dtype, int64_t rows, void* stream) {
+    if (!p || !x || !xm || !rows_ok(rows)) return SFNO_EINVAL;
+    return irfft_launch(p->fft, xm, x, x_dtype, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
 }
 
 extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, float* spec, int64_t rows, void* stream) {
@@ -189,18 +195,18 @@ extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec
     return legendre_fold_launch(false, a, p->inv.n_work, (hipStream_t)stream);
 }
 
-extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const float* x, float* spec, int64_t rows, void* workspace,
+extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const void* x, int x_dtype, float* spec, int64_t rows, void* workspace,
                                  size_t workspace_bytes, void* stream) {
     if (!p || !x || !spec || !rows_ok(rows)) return SFNO_EINVAL;
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
-    int rc = sfno_rfft(p, x, w.xm, rows, stream);
+    int rc = sfno_rfft(p, x, x_dtype, w.xm, rows, stream);
     if (rc != SFNO_OK) return rc;
     return sfno_legendre_analysis(p, w.xm, spec, rows, stream);
 }
 
-extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, float* x, int64_t rows, void* workspace,
+extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, void* x, int x_dtype, int64_t rows, void* workspace,
                                   size_t workspace_bytes, void* stream) {
     if (!p || !x || !spec || !rows_ok(rows)) return SFNO_EINVAL;
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
@@ -208,7 +214,7 @@ extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, flo
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     int rc = sfno_legendre_synthesis(p, spec, w.xm, rows, stream);
     if (rc != SFNO_OK) return rc;
-    return sfno_irfft(p, w.xm, x, rows, stream);
+    return sfno_irfft(p, w.xm, x, x_dtype, rows, stream);
 }
 
 extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* coeffs, int64_t rows, void* workspace,
@@ -216,7 +222,7 @@ extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* co
     if (!p || !coeffs || !rows_ok(rows)) return SFNO_EINVAL;
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
-    int rc = sfno_sht_analysis(p, x, w.spec, rows, workspace, workspace_bytes, stream);
+    int rc = sfno_sht_analysis(p, x, SFNO_DTYPE_F32, w.spec, rows, workspace, workspace_bytes, stream);
     if (rc != SFNO_OK) return rc;
     return spectral_to_coeffs_launch(w.spec, reinterpret_cast<float2*>(coeffs), rows, p->lmax, p->mmax,
                                      (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
@@ -230,7 +236,7 @@ extern "C" int sfno_sht_inverse(const sfno_sht_plan* p, const void* coeffs, floa
     int rc = coeffs_to_spectral_launch(reinterpret_cast<const float2*>(coeffs), w.spec, rows, p->lmax, p->mmax,
                                        (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
     if (rc != SFNO_OK) return rc;
-    return sfno_sht_synthesis(p, w.spec, x, rows, workspace, workspace_bytes, stream);
+    return sfno_sht_synthesis(p, w.spec, x, SFNO_DTYPE_F32, rows, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sfno_coeffs_to_spectral(const void* coeffs, float* spec, int64_t rows, int lmax, int mmax, int triangular,

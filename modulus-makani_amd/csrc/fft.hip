@@ -298,9 +298,11 @@ static int pick_pairs(int n) {
     return 0;
 }
 
-int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+int rfft_launch(const FftPlan& p, const void* xv, int x_dtype, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     if (mmax > p.n / 2 + 1 || ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
-    if (fft_fast_supported(p.n)) return fft_fast_launch(false, p, x, xm, rows, nlat, mmax, ld, s);
+    if (fft_fast_supported(p.n)) return fft_fast_launch(false, p, xv, xm, rows, nlat, mmax, ld, x_dtype, s);
+    if (x_dtype != SFNO_DTYPE_F32) return SFNO_EUNSUPPORTED;     // the generic kernels read float only
+    const float* x = reinterpret_cast<const float*>(xv);
     switch (pick_pairs(p.n)) {
         case 4: return rfft_go<4>(p, x, xm, rows, nlat, mmax, ld, s);
         case 2: return rfft_go<2>(p, x, xm, rows, nlat, mmax, ld, s);
@@ -309,10 +311,12 @@ int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int n
     return SFNO_EUNSUPPORTED;
 }
 
-int irfft_launch(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+int irfft_launch(const FftPlan& p, const float* xm, void* xv, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     // orders above nlon/2 are dropped, as torch.fft.irfft(n=nlon) drops surplus input bins
     if (ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
-    if (fft_fast_supported(p.n)) return fft_fast_launch(true, p, xm, x, rows, nlat, mmax, ld, s);
+    if (fft_fast_supported(p.n)) return fft_fast_launch(true, p, xm, xv, rows, nlat, mmax, ld, x_dtype, s);
+    if (x_dtype != SFNO_DTYPE_F32) return SFNO_EUNSUPPORTED;
+    float* x = reinterpret_cast<float*>(xv);
     switch (pick_pairs(p.n)) {
         case 4: return irfft_go<4>(p, xm, x, rows, nlat, mmax, ld, s);
         case 2: return irfft_go<2>(p, xm, x, rows, nlat, mmax, ld, s);

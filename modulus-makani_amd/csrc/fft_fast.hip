@@ -164,6 +164,35 @@ struct Geo {
     }
 };
 
+// Grid-side element type: float (BF16 = false) or bfloat16 (BF16 = true).  The bf16 variants fuse the
+// up-cast before the forward transform and the round-to-nearest-even down-cast after the inverse
+// (the `x.float()` / `x.to(dtype)` passes of makani/models/common/spectral_convolution.py:127,146).
+template <bool BF16>
+__device__ __forceinline__ float4 load4(const void* base, int64_t idx) {
+    if (BF16) {
+        const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(base) + idx);
+        return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                           __uint_as_float(v.y & 0xffff0000u));
+    }
+    return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + idx);
+}
+__device__ __forceinline__ unsigned bf16_rne(float f) {
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;      // NaN stays NaN
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+template <bool BF16>
+__device__ __forceinline__ void store4(void* base, int64_t idx, float4 v) {
+    if (BF16) {
+        uint2 o;
+        o.x = bf16_rne(v.x) | (bf16_rne(v.y) << 16);
+        o.y = bf16_rne(v.z) | (bf16_rne(v.w) << 16);
+        *reinterpret_cast<uint2*>(reinterpret_cast<unsigned short*>(base) + idx) = o;
+    } else {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(base) + idx) = v;
+    }
+}
+
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  All channel groups of one
 // latitude go to the same XCD, back to back, so that the 64-byte pieces they read or write
 // of one order-major row meet in that XCD's L2 as whole cache lines.
@@ -303,8 +332,8 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
 }
 
 // grid = 8 * ceil(nlat/8) * ngroups workgroups, ngroups = ceil((ld/4) / S), see map_block
-template <int N, int R0, int R1, int R2, int S, int FT>
-__global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ x,
+template <int N, int R0, int R1, int R2, int S, int FT, bool BF16>
+__global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const void* __restrict__ x,
                                                        float* __restrict__ xm, int64_t rows, int nlat, int mmax, int ld, int ngroups, float scale) {
     using G = Geo<N, R0, R1, R2>;
     __shared__ __align__(16) float2 z[S * G::PITCH];
@@ -323,8 +352,8 @@ __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict_
             const int64_t r0 = 2 * (int64_t)(pair0 + p);
             a[it] = make_float4(0.f, 0.f, 0.f, 0.f);
             b[it] = a[it];
-            if (e < TOT && r0 < rows) a[it] = *reinterpret_cast<const float4*>(x + (r0 * nlat + lat) * N + 4 * i4);
-            if (e < TOT && r0 + 1 < rows) b[it] = *reinterpret_cast<const float4*>(x + ((r0 + 1) * nlat + lat) * N + 4 * i4);
+            if (e < TOT && r0 < rows) a[it] = load4<BF16>(x, (r0 * nlat + lat) * N + 4 * i4);
+            if (e < TOT && r0 + 1 < rows) b[it] = load4<BF16>(x, ((r0 + 1) * nlat + lat) * N + 4 * i4);
         }
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
@@ -355,9 +384,9 @@ __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict_
     }
 }
 
-template <int N, int R0, int R1, int R2, int S, int FT>
+template <int N, int R0, int R1, int R2, int S, int FT, bool BF16>
 __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ xm,
-                                                        float* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups) {
+                                                        void* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups) {
     using G = Geo<N, R0, R1, R2>;
     static_assert(N % 2 == 0, "even length");
     __shared__ __align__(16) float2 z[S * G::PITCH];
@@ -411,8 +440,8 @@ __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict
                 const int64_t r0 = 2 * (int64_t)(pair0 + p);
                 const float4* src = reinterpret_cast<const float4*>(z + p * G::PITCH + 4 * i4);
                 const float4 u0 = src[0], u1 = src[1];
-                if (r0 < rows) *reinterpret_cast<float4*>(x + (r0 * nlat + lat) * N + 4 * i4) = make_float4(u0.x, u0.z, u1.x, u1.z);
-                if (r0 + 1 < rows) *reinterpret_cast<float4*>(x + ((r0 + 1) * nlat + lat) * N + 4 * i4) = make_float4(u0.y, u0.w, u1.y, u1.w);
+                if (r0 < rows) store4<BF16>(x, (r0 * nlat + lat) * N + 4 * i4, make_float4(u0.x, u0.z, u1.x, u1.z));
+                if (r0 + 1 < rows) store4<BF16>(x, ((r0 + 1) * nlat + lat) * N + 4 * i4, make_float4(u0.y, u0.w, u1.y, u1.w));
             }
         }
     }
@@ -430,8 +459,8 @@ const FastEntry* find_fast(int n) {
     return nullptr;
 }
 
-template <int N, int R0, int R1, int R2>
-int go_fast(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+template <int N, int R0, int R1, int R2, bool BF16>
+int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     constexpr int S = (N >= 1024) ? 4 : 8;
     constexpr int FT = (S * N >= 4096) ? 512 : 256;     // threads per workgroup
     const int ngroups = (ld / 4 + S - 1) / S;
@@ -440,9 +469,11 @@ int go_fast(bool inverse, const FftPlan& p, const float* in, float* out, int64_t
     dim3 grid((unsigned)nblocks);
     if (!inverse) {
         float scale = (float)(kTwoPi / (double)N);
-        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S, FT>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups, scale);
+        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, reinterpret_cast<float*>(out),
+                           rows, nlat, mmax, ld, ngroups, scale);
     } else {
-        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, FT>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, rows, nlat, mmax, ld, ngroups);
+        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, reinterpret_cast<const float*>(in), out,
+                           rows, nlat, mmax, ld, ngroups);
     }
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
@@ -474,13 +505,21 @@ int fft_fast_plan_init(FftPlan& p) {
     return SFNO_OK;
 }
 
-int fft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
+                    hipStream_t s) {
+    const bool bf = grid_dtype == SFNO_DTYPE_BF16;
+    if (!bf && grid_dtype != SFNO_DTYPE_F32) return SFNO_EUNSUPPORTED;
+#define FF_CASE(N_, A_, B_, C_)                                                                          \
+    case N_:                                                                                             \
+        return bf ? go_fast<N_, A_, B_, C_, true>(inverse, p, in, out, rows, nlat, mmax, ld, s)           \
+                  : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, s);
     switch (p.n) {
-        case 1440: return go_fast<1440, 16, 10, 9>(inverse, p, in, out, rows, nlat, mmax, ld, s);
-        case 480: return go_fast<480, 10, 16, 3>(inverse, p, in, out, rows, nlat, mmax, ld, s);
-        case 64: return go_fast<64, 8, 8, 1>(inverse, p, in, out, rows, nlat, mmax, ld, s);
-        case 180: return go_fast<180, 4, 5, 9>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+        FF_CASE(1440, 16, 10, 9)
+        FF_CASE(480, 10, 16, 3)
+        FF_CASE(64, 8, 8, 1)
+        FF_CASE(180, 4, 5, 9)
     }
+#undef FF_CASE
     return SFNO_EUNSUPPORTED;
 }
 

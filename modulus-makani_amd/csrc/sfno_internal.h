@@ -79,14 +79,15 @@ struct FftPlan {
 };
 bool fft_fast_supported(int n);
 int fft_fast_plan_init(FftPlan& p);
-int fft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int64_t rows, int nlat, int mmax, int ld,
+// grid_dtype: element type of the grid-side tensor (SFNO_DTYPE_*); the Fourier side is always float
+int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
                     hipStream_t s);
 int fft_plan_init(FftPlan& p, int n);
 void fft_plan_free(FftPlan& p);
 // x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon
-int rfft_launch(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+int rfft_launch(const FftPlan& p, const void* x, int x_dtype, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
 // xm [mmax][nlat][ld] -> x [rows][nlat][nlon]
-int irfft_launch(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+int irfft_launch(const FftPlan& p, const float* xm, void* x, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
 
 // ---- layout passes (layout.hip) ----------------------------------------------------------
 int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri,

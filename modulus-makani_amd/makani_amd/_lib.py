@@ -14,6 +14,7 @@ GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2}
 NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
 DIR_FORWARD, DIR_INVERSE = 1, 2
 COMPUTE_FP32, COMPUTE_BF16 = 0, 1
+DTYPE_F32, DTYPE_BF16 = 0, 1
 
 
 class SfnoError(RuntimeError):
@@ -42,10 +43,11 @@ def _load():
         "sfno_sht_workspace_bytes": (sz, [vp, i64]),
         "sfno_sht_forward": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_inverse": (i32, [vp, vp, vp, i64, vp, sz, vp]),
-        "sfno_sht_analysis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
-        "sfno_sht_synthesis": (i32, [vp, vp, vp, i64, vp, sz, vp]),
-        "sfno_rfft": (i32, [vp, vp, vp, i64, vp]),
-        "sfno_irfft": (i32, [vp, vp, vp, i64, vp]),
+        "sfno_sht_io_dtype_supported": (i32, [vp, i32]),
+        "sfno_sht_analysis": (i32, [vp, vp, i32, vp, i64, vp, sz, vp]),
+        "sfno_sht_synthesis": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),
+        "sfno_rfft": (i32, [vp, vp, i32, vp, i64, vp]),
+        "sfno_irfft": (i32, [vp, vp, vp, i32, i64, vp]),
         "sfno_legendre_analysis": (i32, [vp, vp, vp, i64, vp]),
         "sfno_legendre_synthesis": (i32, [vp, vp, vp, i64, vp]),
         "sfno_fourier_elems": (i64, [vp, i64]),

@@ -183,15 +183,21 @@ class RealSHT(_SHTBase):
         return out
 
     def analysis(self, x):
-        """x [..., nlat, nlon] -> spectral-layout float32 [mmax, lmax, ld] (internal fast path)."""
+        """x [..., nlat, nlon] (float32, or bfloat16 widened inside the FFT kernel) -> spectral-layout float32 [mmax, lmax, ld]."""
         assert x.shape[-2] == self.nlat
         assert x.shape[-1] == self.nlon
-        x = _as_fp32_rows(x, "grid")
-        rows = int(np.prod(x.shape[:-2])) if x.dim() > 2 else 1
         plan = self.plan(x.device)
+        dt = _lib.DTYPE_F32
+        if x.dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16):
+            if x.requires_grad and torch.is_grad_enabled():
+                raise NotImplementedError("backward through the HIP spherical harmonic transforms is not implemented")
+            x, dt = x.contiguous(), _lib.DTYPE_BF16
+        else:
+            x = _as_fp32_rows(x, "grid")
+        rows = int(np.prod(x.shape[:-2])) if x.dim() > 2 else 1
         spec = torch.empty(self.spectral_shape(rows), dtype=torch.float32, device=x.device)
         ws, nbytes = self.workspace(plan, rows, x.device)
-        check(lib.sfno_sht_analysis(plan.handle, _ptr(x), _ptr(spec), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_analysis")
+        check(lib.sfno_sht_analysis(plan.handle, _ptr(x), dt, _ptr(spec), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_analysis")
         return spec
 
 
@@ -220,12 +226,14 @@ class InverseRealSHT(_SHTBase):
         check(lib.sfno_sht_inverse(plan.handle, _ptr(x), _ptr(out), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_inverse")
         return out
 
-    def synthesis(self, spec, lead):
-        """spectral-layout float32 [mmax, lmax, ld] -> x [*lead, nlat, nlon] (internal fast path)."""
+    def synthesis(self, spec, lead, dtype=torch.float32):
+        """spectral-layout float32 [mmax, lmax, ld] -> x [*lead, nlat, nlon]; dtype bfloat16 rounds inside the FFT kernel."""
         rows = int(np.prod(lead)) if len(lead) else 1
         assert tuple(spec.shape) == self.spectral_shape(rows) and spec.dtype == torch.float32 and spec.is_contiguous()
         plan = self.plan(spec.device)
-        out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.float32, device=spec.device)
+        fused = dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16)
+        out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.bfloat16 if fused else torch.float32, device=spec.device)
         ws, nbytes = self.workspace(plan, rows, spec.device)
-        check(lib.sfno_sht_synthesis(plan.handle, _ptr(spec), _ptr(out), rows, _ptr(ws), nbytes, _stream_ptr(spec.device)), "sfno_sht_synthesis")
-        return out
+        check(lib.sfno_sht_synthesis(plan.handle, _ptr(spec), _ptr(out), _lib.DTYPE_BF16 if fused else _lib.DTYPE_F32, rows, _ptr(ws), nbytes,
+                                     _stream_ptr(spec.device)), "sfno_sht_synthesis")
+        return out if out.dtype == dtype else out.to(dtype)

@@ -69,17 +69,20 @@ class SpectralConv(nn.Module):
     def forward(self, x):
         dtype = x.dtype
         residual = x
-        x = x.float()
         B, C, H, W = x.shape
 
         if self._fused:
-            # the transforms and the contraction all work on float32 regardless of autocast
-            spec = self.forward_transform.analysis(x)
+            # The transforms and the contraction work in float32 regardless of autocast.  A bf16 input is
+            # widened while the FFT kernel loads it and the output is rounded while it is stored: the
+            # same values as the reference's x.float() ... x.to(dtype) without the two full-tensor passes.
+            fuse_cast = dtype == torch.bfloat16 and not hasattr(self, "bias")
+            spec = self.forward_transform.analysis(x if dtype == torch.bfloat16 else x.float())
             if self.scale_residual:
-                residual = self.inverse_transform.synthesis(spec, (B, C)).to(dtype)
+                residual = self.inverse_transform.synthesis(spec, (B, C), dtype=dtype if dtype == torch.bfloat16 else torch.float32).to(dtype)
             spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=True)
-            x = self.inverse_transform.synthesis(spec, (B, self.out_channels))
+            x = self.inverse_transform.synthesis(spec, (B, self.out_channels), dtype=dtype if fuse_cast else torch.float32)
         else:
+            x = x.float()
             with torch.autocast(device_type="cuda", enabled=False):
                 x = self.forward_transform(x).contiguous()
                 if self.scale_residual:

@@ -127,3 +127,23 @@ def test_inverse_surplus_orders(lib_built):
     assert rel_l2(got.cpu().numpy(), ref) < TOL
     with pytest.raises(ValueError):
         ma.RealSHT(16, 32, lmax=32, mmax=33, grid="legendre-gauss")
+
+
+@pytest.mark.parametrize("nlat,nlon,lmax,mmax,grid", [(32, 64, 20, 21, "equiangular"), (40, 480, 40, 41, "legendre-gauss"), (12, 30, 10, 9, "legendre-gauss")])
+def test_bf16_grid_io_equals_cast_then_transform(lib_built, nlat, nlon, lmax, mmax, grid):
+    """A bf16 field transformed directly equals the transform of its float32 widening, bit for bit; a bf16 output
+    equals the float32 output rounded to nearest even (the reference's x.float() / x.to(dtype) around the transforms)."""
+    import makani_amd as ma
+
+    torch.manual_seed(7)
+    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
+    xb = torch.randn(3, 5, nlat, nlon).to(torch.bfloat16).cuda()
+    s_direct = sht.analysis(xb)
+    s_cast = sht.analysis(xb.float())
+    # entries with l < m (and the channel padding) are never written: compare the defined part
+    valid = (torch.arange(s_cast.shape[1])[None, :] >= torch.arange(s_cast.shape[0])[:, None]).cuda()
+    assert torch.equal(s_direct[..., : 2 * 15][valid], s_cast[..., : 2 * 15][valid])
+    y32 = isht.synthesis(s_cast, (3, 5))
+    yb = isht.synthesis(s_cast, (3, 5), dtype=torch.bfloat16)
+    assert yb.dtype == torch.bfloat16 and torch.equal(yb, y32.to(torch.bfloat16))

@@ -259,15 +259,23 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
     if (!out) return SFNO_EINVAL;
     *out = nullptr;
     if (I < 1 || O < 1 || L < 1) return SFNO_EINVAL;
-    if (compute != SFNO_COMPUTE_FP32) return SFNO_EUNSUPPORTED;
+    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16) return SFNO_EUNSUPPORTED;
+    // the bf16 kernel reads activation rows in groups of four floats
+    if (compute == SFNO_COMPUTE_BF16 && (2 * I) % 4 != 0) return SFNO_EUNSUPPORTED;
     sfno_dhconv_weights* w = new (std::nothrow) sfno_dhconv_weights();
     if (!w) return SFNO_ENOMEM;
     w->I = I; w->O = O; w->L = L; w->compute = compute;
     if (hipGetDevice(&w->device) != hipSuccess) { delete w; return SFNO_EHIP; }
-    w->nob = (2 * O + DH_COLS - 1) / DH_COLS;
-    w->nc = (2 * I + PG_KC - 1) / PG_KC;
-    // 8 x 64 complex numbers per (degree, column block, chunk)
-    const size_t bytes = sizeof(float) * 1024 * (size_t)L * w->nob * w->nc;
+    size_t bytes;
+    if (compute == SFNO_COMPUTE_BF16) {
+        w->nob = (2 * O + 255) / 256;
+        w->nc = (2 * I + 31) / 32;
+        bytes = 8192 * (size_t)L * w->nob * w->nc;          // 128 x 16 complex bf16 per (degree, column block, chunk)
+    } else {
+        w->nob = (2 * O + DH_COLS - 1) / DH_COLS;
+        w->nc = (2 * I + PG_KC - 1) / PG_KC;
+        bytes = sizeof(float) * 1024 * (size_t)L * w->nob * w->nc;   // 8 x 64 complex fp32
+    }
     if (hipMalloc((void**)&w->d_W, bytes) != hipSuccess) { delete w; return SFNO_ENOMEM; }
     *out = w;
     return SFNO_OK;
@@ -275,6 +283,8 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
 
 extern "C" int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream) {
     if (!w || !weight) return SFNO_EINVAL;
+    if (w->compute == SFNO_COMPUTE_BF16)
+        return dhconv_pack_bf16_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, (hipStream_t)stream);
     return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, (hipStream_t)stream);
 }
 
@@ -302,6 +312,7 @@ extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* s
     a.ld_out = (int)sfno_spectral_ld((int64_t)batch * w->O);
     a.nob = w->nob;
     a.nc = w->nc;
+    if (w->compute == SFNO_COMPUTE_BF16) return dhconv_bf16_launch(a, (hipStream_t)stream);
     return dhconv_launch(a, (hipStream_t)stream);
 }
 

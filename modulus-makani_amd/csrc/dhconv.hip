@@ -161,6 +161,165 @@ int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, hipS
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
+// ---- bf16 variant ---------------------------------------------------------------------------------------
+// Same decomposition on v_mfma_f32_32x32x16_bf16 (fp32 accumulate): activations are rounded to bf16 (nearest
+// even) in registers as they arrive, weights are stored as complex bf16 and expanded to the real embedding by
+// two bit operations per word while they are copied to LDS.  K is walked in chunks of 32 i'; lane group kg of a
+// wavefront takes i' = 32c + 16kg + 8s .. +7 in k-step s, on both operands, so that every lane reads 64
+// contiguous bytes of its activation row and 16 contiguous bytes of a weight column per step.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+constexpr int DHB_COLS = 256;          // output columns o' per workgroup
+constexpr int DHB_KC = 32;             // i' per chunk
+
+__device__ __forceinline__ bf16x8 to_bf16x8(f4 a, f4 b) {
+    bf16x8 v;
+    v[0] = (__bf16)a[0]; v[1] = (__bf16)a[1]; v[2] = (__bf16)a[2]; v[3] = (__bf16)a[3];
+    v[4] = (__bf16)b[0]; v[5] = (__bf16)b[1]; v[6] = (__bf16)b[2]; v[7] = (__bf16)b[3];
+    return v;
+}
+
+// grid = (8 * ceil(L/8) * nob, row groups of 128), nob = ceil(2*O / 256); requires 2*I % 8 == 0
+__global__ __launch_bounds__(256, 2) void dhconv_bf16_kernel(DhconvArgs a) {
+    constexpr int NT = DHB_COLS / 32;                // 8 column tiles per wavefront
+    constexpr int PITCH = DHB_KC + 8;                // bf16 elements per LDS row (80 bytes: 16-byte reads of 16 lanes hit distinct banks)
+    __shared__ __align__(16) unsigned short ws[2][DHB_COLS][PITCH];
+
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
+    if (lidx >= a.L) return;
+    const int l = a.L - 1 - lidx;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
+    const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;
+    const int r0 = blockIdx.y * 128;
+    if (r0 >= ncols) return;
+    const bool active = r0 + 32 * wave < ncols;
+    const int nc = a.nc;                                           // chunks of 32 i'
+    const int kg = lane >> 5, cl = lane & 31;
+
+    const int n = min(r0 + 32 * wave + cl, ncols - 1);
+    const int mm = n / a.B, bb = n - mm * a.B;
+    const float* xrow = a.X + ((int64_t)mm * a.L + l) * a.ld_in + (int64_t)bb * a.I2;
+    // packed weights of (l, ob): nc chunks of 128 (o) x 16 (i) complex bf16 = 8 KiB, two 16-byte pieces per thread
+    const u4* wp = reinterpret_cast<const u4*>(a.W) + ((int64_t)l * a.nob + ob) * nc * 512 + tid;
+
+    floatx16 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+
+    // my 16 activations of the chunk: i' = 32c + 16kg .. +15 (clamped in groups of four; weights are zero past 2*I)
+    auto x_load = [&](int c, f4 (&xr)[4]) {
+        const int k = DHB_KC * c + 16 * kg;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xr[j] = *reinterpret_cast<const f4*>(xrow + min(k + 4 * j, a.I2 - 4));
+    };
+    // piece e (16 bytes = 4 complex = 8 i') of the chunk: o = e / 4, i-group g = e % 4; it becomes 16 bytes of row 2o
+    // (re, -im, ...) and 16 bytes of row 2o+1 (im, re, ...)
+    auto w_store = [&](int buf, const u4 (&w)[2]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = tid + 256 * u, o = e >> 2, g = e & 3;
+            const u4 even = w[u] ^ 0x80000000u;
+            const u4 odd = (w[u] >> 16) | (w[u] << 16);
+            *reinterpret_cast<u4*>(&ws[buf][2 * o][8 * g]) = even;
+            *reinterpret_cast<u4*>(&ws[buf][2 * o + 1][8 * g]) = odd;
+        }
+    };
+    auto compute = [&](int buf, const f4 (&xr)[4]) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const bf16x8 xa = to_bf16x8(xr[2 * s], xr[2 * s + 1]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const bf16x8 wb = *reinterpret_cast<const bf16x8*>(&ws[buf][32 * t + cl][16 * kg + 8 * s]);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa, wb, acc[t], 0, 0, 0);
+            }
+        }
+    };
+
+    f4 xcur[4], xnext[4];
+    u4 wnext[2];
+    x_load(0, xcur);
+    wnext[0] = wp[0];
+    wnext[1] = wp[256];
+    w_store(0, wnext);
+    __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0)
+    __syncthreads();
+    for (int c = 0; c < nc; ++c) {
+        const int buf = c & 1;
+        const bool more = c + 1 < nc;
+        if (more) {
+            wnext[0] = wp[(int64_t)(c + 1) * 512];
+            wnext[1] = wp[(int64_t)(c + 1) * 512 + 256];
+            x_load(c + 1, xnext);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (active) compute(buf, xcur);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) w_store(buf ^ 1, wnext);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xcur[j] = xnext[j];
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int nn = r0 + 32 * wave + 8 * (v >> 2) + 4 * kg + (v & 3);
+        if (nn >= ncols) continue;
+        const int m2 = nn / a.B, b2 = nn - m2 * a.B;
+        float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int oc = DHB_COLS * ob + 32 * t + cl;
+            if (oc < a.O2) orow[oc] = acc[t][v];
+        }
+    }
+}
+
+// packed[l][ob][c][o (128)][i (16)] = bf16(re) | bf16(im) << 16 of w[16c + i][128 ob + o][l], zero outside the weight
+__global__ __launch_bounds__(256) void dhconv_pack_bf16_kernel(const float2* __restrict__ w, unsigned int* __restrict__ packed, int I, int O, int L,
+                                                               int nob, int nc) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)L * nob * nc * 2048;
+    if (idx >= total) return;
+    const int ii = (int)(idx & 15), o = (int)((idx >> 4) & 127);
+    int64_t rem = idx >> 11;
+    const int c = (int)(rem % nc);
+    rem /= nc;
+    const int ob = (int)(rem % nob), l = (int)(rem / nob);
+    const int i = 16 * c + ii, oo = 128 * ob + o;
+    unsigned int v = 0;
+    if (i < I && oo < O) {
+        const float2 z = w[((int64_t)i * O + oo) * L + l];
+        const __bf16 re = (__bf16)z.x, im = (__bf16)z.y;
+        v = (unsigned int)__builtin_bit_cast(unsigned short, re) | ((unsigned int)__builtin_bit_cast(unsigned short, im) << 16);
+    }
+    packed[idx] = v;
+}
+
+int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, hipStream_t s) {
+    const int nob = (2 * O + DHB_COLS - 1) / DHB_COLS, nc = (2 * I + DHB_KC - 1) / DHB_KC;
+    const int64_t total = (int64_t)L * nob * nc * 2048;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_pack_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s) {
+    const int64_t rows_max = (int64_t)a.M * a.B;
+    if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
+    if (a.I2 % 4 != 0 || a.ld_in % 4 != 0) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
+    hipLaunchKernelGGL(dhconv_bf16_kernel, grid, dim3(256), 0, s, a);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
 int dhconv_launch(const DhconvArgs& a, hipStream_t s) {
     const int64_t rows_max = (int64_t)a.M * a.B;
     if (rows_max <= 0 || a.L <= 0) return SFNO_OK;

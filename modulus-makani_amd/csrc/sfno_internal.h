@@ -49,6 +49,9 @@ struct DhconvArgs {
     int nob, nc;                   // column blocks of DH_COLS over 2*O, K chunks of 16 over 2*I
 };
 int dhconv_launch(const DhconvArgs& a, hipStream_t s);
+// bf16 MFMA variant: 256 output columns per workgroup, K chunks of 32, weights packed as complex bf16
+int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s);
+int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, hipStream_t s);
 
 // ---- host-side table construction (tables.cpp) -----------------------------------------
 int quadrature(int grid, int nlat, double* theta, double* w);

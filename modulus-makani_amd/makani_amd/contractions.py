@@ -15,13 +15,14 @@ from ._lib import lib, check
 class PackedWeights:
     """Device handle holding a SpectralConv weight packed as per-degree MFMA operand stream."""
 
-    def __init__(self, in_channels, out_channels, lmax, device):
+    def __init__(self, in_channels, out_channels, lmax, device, compute="fp32"):
         self.handle = ctypes.c_void_p()
         self.shape = (in_channels, out_channels, lmax)
         self.device = torch.device(device)
+        self.compute = compute
         self.stamp = None
         with torch.cuda.device(self.device):
-            check(lib.sfno_dhconv_weights_create(in_channels, out_channels, lmax, _lib.COMPUTE_FP32, ctypes.byref(self.handle)), "sfno_dhconv_weights_create")
+            check(lib.sfno_dhconv_weights_create(in_channels, out_channels, lmax, COMPUTE[compute], ctypes.byref(self.handle)), "sfno_dhconv_weights_create")
 
     def refresh(self, weight):
         """Re-pack if the parameter changed (in-place updates bump ``_version``)."""
@@ -42,27 +43,32 @@ class PackedWeights:
             self.handle = None
 
 
-# id(tensor) -> (weak reference to the tensor, PackedWeights); tensors compare element-wise,
+# arithmetic of the contraction: fp32 MFMA, or bf16 MFMA inputs with fp32 accumulation
+COMPUTE = {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16}
+
+# (id(tensor), compute) -> (weak reference to the tensor, PackedWeights); tensors compare element-wise,
 # so they cannot key a WeakKeyDictionary directly
 _cache = {}
 
 
-def packed_for(weight):
+def packed_for(weight, compute="fp32"):
     """Packed handle for a weight tensor, cached per tensor object and refreshed when it changes."""
     if weight.device.type != "cuda":
         raise RuntimeError("the dhconv kernel runs on a HIP device only")
-    key = id(weight)
+    if compute not in COMPUTE:
+        raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32' or 'bf16'")
+    key = (id(weight), compute)
     hit = _cache.get(key)
     p = hit[1] if hit is not None and hit[0]() is weight else None
     if p is None or p.device != weight.device or p.shape != tuple(weight.shape):
-        p = PackedWeights(weight.shape[0], weight.shape[1], weight.shape[2], weight.device)
+        p = PackedWeights(weight.shape[0], weight.shape[1], weight.shape[2], weight.device, compute)
         _cache[key] = (weakref.ref(weight, lambda _, k=key: _cache.pop(k, None)), p)
     return p.refresh(weight)
 
 
-def dhconv_spectral(spec_in, weight, batch, mmax, triangular=True):
+def dhconv_spectral(spec_in, weight, batch, mmax, triangular=True, compute="fp32"):
     """Spectral-layout contraction: [mmax, L, ld(batch*I)] -> [mmax, L, ld(batch*O)]."""
-    pw = packed_for(weight)
+    pw = packed_for(weight, compute)
     I, O, L = pw.shape
     ld_out = int(lib.sfno_spectral_ld(batch * O))
     out = torch.empty((mmax, L, ld_out), dtype=torch.float32, device=spec_in.device)
@@ -76,7 +82,7 @@ def dhconv_spectral(spec_in, weight, batch, mmax, triangular=True):
     return out
 
 
-def _contract_dhconv(ac: torch.Tensor, bc: torch.Tensor, triangular: bool = False) -> torch.Tensor:
+def _contract_dhconv(ac: torch.Tensor, bc: torch.Tensor, triangular: bool = False, compute: str = "fp32") -> torch.Tensor:
     """einsum("bixy,iox->boxy") on complex64 tensors (contractions.py:130-136)."""
     if ac.dim() != 4 or bc.dim() != 3 or ac.shape[1] != bc.shape[0] or ac.shape[2] != bc.shape[2]:
         raise RuntimeError(f"dhconv: shapes {tuple(ac.shape)} and {tuple(bc.shape)} do not match 'bixy,iox->boxy'")
@@ -87,7 +93,7 @@ def _contract_dhconv(ac: torch.Tensor, bc: torch.Tensor, triangular: bool = Fals
     ac = ac.contiguous()
     B, I, L, M = ac.shape
     O = bc.shape[1]
-    pw = packed_for(bc)
+    pw = packed_for(bc, compute)
     out = torch.empty((B, O, L, M), dtype=torch.complex64, device=ac.device)
     if out.numel() == 0:
         return out

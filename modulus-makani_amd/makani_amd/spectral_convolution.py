@@ -14,8 +14,11 @@ from .sht import RealSHT, InverseRealSHT
 class SpectralConv(nn.Module):
     """Spectral convolution on the sphere: SHT -> per-degree complex channel mix -> inverse SHT."""
 
-    def __init__(self, forward_transform, inverse_transform, in_channels, out_channels, operator_type="diagonal", separable=False, bias=False, gain=1.0):
+    def __init__(self, forward_transform, inverse_transform, in_channels, out_channels, operator_type="diagonal", separable=False, bias=False, gain=1.0,
+                 compute="fp32"):
         super().__init__()
+        # compute = "bf16" runs the channel mix on bf16 MFMA (fp32 accumulate); the reference and the default stay fp32
+        self.compute = compute
         self.forward_transform = forward_transform
         self.inverse_transform = inverse_transform
         self.in_channels = in_channels
@@ -79,7 +82,7 @@ class SpectralConv(nn.Module):
             spec = self.forward_transform.analysis(x if dtype == torch.bfloat16 else x.float())
             if self.scale_residual:
                 residual = self.inverse_transform.synthesis(spec, (B, C), dtype=dtype if dtype == torch.bfloat16 else torch.float32).to(dtype)
-            spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=True)
+            spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=True, compute=self.compute)
             x = self.inverse_transform.synthesis(spec, (B, self.out_channels), dtype=dtype if fuse_cast else torch.float32)
         else:
             x = x.float()

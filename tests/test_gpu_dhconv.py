@@ -83,3 +83,24 @@ def test_spectral_conv_matches_oracle(lib_built, fwd, inv, B, C, O):
     assert y.shape == y_ref.shape and res.shape == res_ref.shape
     assert rel_l2(y.cpu().numpy(), y_ref) < TOL
     assert rel_l2(res.cpu().numpy(), res_ref) < TOL
+
+
+@pytest.mark.parametrize("B,I,O,L,M", [(1, 4, 2, 4, 5), (2, 8, 8, 6, 7), (1, 64, 48, 40, 41), (3, 18, 6, 12, 9), (1, 384, 384, 24, 25), (4, 24, 200, 70, 71)])
+def test_contract_dhconv_bf16(lib_built, B, I, O, L, M):
+    """bf16 MFMA variant (inputs rounded to bf16, fp32 accumulation): relative L2 <= 1e-2 against the float64 oracle."""
+    import makani_amd as ma
+
+    print(f"case dhconv bf16 B={B} I={I} O={O} L={L} M={M}", flush=True)
+    torch.manual_seed(2)
+    x = torch.randn(B, I, L, M, dtype=torch.complex64)
+    w = torch.randn(I, O, L, dtype=torch.complex64) / np.sqrt(I)
+    got = ma._contract_dhconv(x.cuda(), w.cuda(), compute="bf16")
+    torch.cuda.synchronize()
+    ref = dhconv(x.numpy().astype(np.complex128), w.numpy().astype(np.complex128))
+    err = rel_l2(got.cpu().numpy(), ref)
+    assert err < 1e-2
+    # and it really is a reduced-precision path: exact bf16 rounding of the inputs reproduces it much more closely
+    xb = torch.view_as_complex(torch.view_as_real(x).to(torch.bfloat16).float())
+    wb = torch.view_as_complex(torch.view_as_real(w).to(torch.bfloat16).float())
+    ref_b = dhconv(xb.numpy().astype(np.complex128), wb.numpy().astype(np.complex128))
+    assert rel_l2(got.cpu().numpy(), ref_b) < 1e-5

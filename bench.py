@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
+    ap.add_argument("--compute", default="fp32", choices=["fp32", "bf16"],
+                    help="arithmetic of the Legendre and dhconv contractions: fp32 MFMA (reference precision) or bf16 MFMA inputs with fp32 accumulation")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--yardstick", action="store_true",
                     help="also run one plain 256 MiB elementwise copy (mul by 1): the known-size reference for FETCH_SIZE/WRITE_SIZE runs")
@@ -130,8 +132,8 @@ def bench_sht_pair(args):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     nlat, nlon, lmax, mmax, grid, C = 721, 1440, 721, 721, "equiangular", 73
-    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
-    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid)
+    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute=args.compute)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute=args.compute)
     x = make_fields(isht, C, dev)
     torch.cuda.synchronize()
 
@@ -191,7 +193,7 @@ def bench_sht_pair(args):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32" if args.compute == "fp32" else "bf16 MFMA inputs, f32 accumulate (FFT f32)",
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: RealSHT + InverseRealSHT, equiangular 721x1440, lmax=mmax=721, batch 1, 73 channels, "
@@ -231,9 +233,9 @@ def bench_spectral_block(args):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     nlat, nlon, L, M, C = 241, 480, 241, 241, 384
-    sht = ma.RealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss")
-    isht = ma.InverseRealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss")
-    conv = ma.SpectralConv(sht, isht, C, C, operator_type="dhconv").to(dev)
+    sht = ma.RealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss", compute=args.compute)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=L, mmax=M, grid="legendre-gauss", compute=args.compute)
+    conv = ma.SpectralConv(sht, isht, C, C, operator_type="dhconv", compute=args.compute).to(dev)
     g = torch.Generator().manual_seed(3)
     w = torch.complex(torch.randn(C, C, L, generator=g), torch.randn(C, C, L, generator=g)) / (2.0 ** 0.5) * (1.0 / C) ** 0.5
     with torch.no_grad():
@@ -257,14 +259,15 @@ def bench_spectral_block(args):
         "value": args.steps / dt,
         "unit": "blocks/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.compute == "fp32" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic",
         "config": {"workload": "configs[2]: SHT -> dhconv -> inverse SHT, legendre-gauss 241x480, lmax=mmax=241, batch 1, 384 channels"},
         "useful_TFLOPs_per_step": (dh_flops + 2 * leg_flops) / 1e12,
         "achieved_TFLOPs": (dh_flops + 2 * leg_flops) / (dt / args.steps) / 1e12,
     }
 
 
-def build_sfno8l(dev):
+def build_sfno8l(dev, compute="fp32"):
     """SFNO-linear, 8 layers, embed 384, scale factor 3, 73 channels in/out (config/sfnonet.yaml:24-40,149-174), random init."""
     import torch
     from makani_amd.sfnonet import SphericalFourierNeuralOperatorNet
@@ -272,15 +275,16 @@ def build_sfno8l(dev):
     torch.manual_seed(4)
     net = SphericalFourierNeuralOperatorNet(inp_shape=(721, 1440), out_shape=(721, 1440), scale_factor=3, inp_chans=73, out_chans=73,
                                             embed_dim=384, num_layers=8, use_mlp=True, mlp_ratio=2.0, activation_function="gelu",
-                                            normalization_layer="instance_norm", big_skip=True, operator_type="dhconv", filter_type="linear")
+                                            normalization_layer="instance_norm", big_skip=True, operator_type="dhconv", filter_type="linear",
+                                            spectral_compute=compute)
     return net.to(dev).eval()
 
 
-def time_sfno_forward(batch, iters, warmup, dev):
+def time_sfno_forward(batch, iters, warmup, dev, compute="fp32"):
     """Median forward time (ms) of the SFNO-8L under bf16 autocast, inference mode, HIP events."""
     import torch
 
-    net = build_sfno8l(dev)
+    net = build_sfno8l(dev, compute)
     x = torch.randn(batch, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
     times = []
     with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
@@ -304,10 +308,11 @@ def bench_sfno8l(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    med, best, _, _ = time_sfno_forward(1, max(args.steps, 5), args.warmup, dev)
+    med, best, _, _ = time_sfno_forward(1, max(args.steps, 5), args.warmup, dev, args.compute)
     return {
         "metric": "SFNO-L8 fwd ms/sample", "value": med, "unit": "ms/sample", "n_gpus": 1, "steps": max(args.steps, 5), "warmup": args.warmup,
-        "ms_per_step": med, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 pointwise / f32 spectral",
+        "ms_per_step": med, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 pointwise / f32 spectral" if args.compute == "fp32" else "bf16 pointwise / bf16-MFMA spectral contractions",
         "data": "synthetic",
         "config": {"workload": "configs[3]: SFNO-linear 8 layers, embed 384, scale factor 3 (721x1440 -> 240x480), 73 channels, batch 1, "
                                "bf16 autocast forward, random-init weights, N(0,1) inputs"},
@@ -321,7 +326,7 @@ def bench_rollout(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    net = build_sfno8l(dev)
+    net = build_sfno8l(dev, args.compute)
     x0 = torch.randn(4, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
     nsteps = 12
     with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):

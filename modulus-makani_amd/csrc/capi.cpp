@@ -33,7 +33,7 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, analysis ? 0 : 1, p.csphase);
     std::vector<float> packed;
     std::vector<int64_t> aoff;
-    pack_legendre_fold(gen, quad_w, analysis, packed, aoff);
+    pack_legendre_fold(gen, quad_w, analysis, p.compute == SFNO_COMPUTE_BF16, packed, aoff);
     // a workgroup covers two 32-row blocks of each parity
     const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
@@ -51,7 +51,7 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     std::vector<int2> work;
     build_worklist(nrb, cost, work, 2);
     t.n_work = (int)work.size();
-    t.n_blocks = (int64_t)(packed.size() / PG_BLOCK_FLOATS);
+    t.n_blocks = (int64_t)(packed.size() / (p.compute == SFNO_COMPUTE_BF16 ? PG_BLOCK_FLOATS / 2 : PG_BLOCK_FLOATS));
     int rc;
     if ((rc = upload(&t.d_A, packed)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_aoff, aoff)) != SFNO_OK) return rc;
@@ -127,7 +127,7 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if ((directions & SFNO_DIR_FORWARD) && mmax > nlon / 2 + 1) return SFNO_EINVAL;
     if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
     if (!(directions & (SFNO_DIR_FORWARD | SFNO_DIR_INVERSE))) return SFNO_EINVAL;
-    if (compute != SFNO_COMPUTE_FP32) return SFNO_EUNSUPPORTED;
+    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16) return SFNO_EUNSUPPORTED;
     sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
     if (!p) return SFNO_ENOMEM;
     p->nlat = nlat; p->nlon = nlon; p->lmax = lmax; p->mmax = mmax;
@@ -184,7 +184,7 @@ extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, f
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->fwd, xm, spec, ld);
-    return legendre_fold_launch(true, a, p->fwd.n_work, (hipStream_t)stream);
+    return legendre_fold_launch(true, p->compute == SFNO_COMPUTE_BF16, a, p->fwd.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec, float* xm, int64_t rows, void* stream) {
@@ -192,7 +192,7 @@ extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv, spec, xm, ld);
-    return legendre_fold_launch(false, a, p->inv.n_work, (hipStream_t)stream);
+    return legendre_fold_launch(false, p->compute == SFNO_COMPUTE_BF16, a, p->inv.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const void* x, int x_dtype, float* spec, int64_t rows, void* workspace,

@@ -17,8 +17,12 @@ namespace sfno {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-template <int NT, bool ANALYSIS>
+// BF16: the table stream holds bf16 (8 per lane and chunk: lane (row, kg) has k = 16c + 8kg .. +7) and the
+// contraction runs on v_mfma_f32_32x32x16_bf16 with the panel values rounded to bf16 (nearest even) as they are
+// read from LDS; accumulation stays fp32.
+template <int NT, bool ANALYSIS, bool BF16>
 __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     constexpr int TN = 32 * NT;
     constexpr int LDQ = TN + ((TN % 64 == 0) ? 32 : 0);
@@ -50,7 +54,9 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     const float* xm_m = (ANALYSIS ? a.Q : a.Out) + (int64_t)m * nlat * ld;     // Fourier panel of order m
     const float* sp_m = (ANALYSIS ? a.Out : a.Q) + (int64_t)m * lmax * ld;     // spectral panel of order m
     // wavefronts without a row block read the head of the table (always at least nc blocks long) and discard it
-    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((active ? a.a_off[2 * m + par] + (int64_t)rb * nc : (int64_t)0) * 128 + lane);
+    // 16 bytes per lane: fp32 blocks are two such pieces per chunk (128 per block), bf16 blocks one (64 per block)
+    constexpr int APB = BF16 ? 64 : 128;
+    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((active ? a.a_off[2 * m + par] + (int64_t)rb * nc : (int64_t)0) * APB + lane);
 
     floatx16 acc[NT];
 #pragma unroll
@@ -112,27 +118,40 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     // One K-chunk of MFMAs.  No branches inside: columns past ld hold zeros in LDS and are
     // masked at the store, so the LDS reads can be issued well ahead of the matrix instructions.
     auto compute = [&](int buf, const f4 (&ar)[2]) {
-        // the panel values of k-step i+1 are read from LDS before the MFMAs of k-step i are issued
-        float qv[2][NT];
-        const float* qbase = &qs[buf][par][kh][cl];
+        if constexpr (BF16) {
+            // ar[0] carries 8 bf16 table values; every column tile gathers its 8 panel values along k
+            const bf16x8 av = __builtin_bit_cast(bf16x8, ar[0]);
+            const float* qbase = &qs[buf][par][8 * kh][cl];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) qv[0][t] = qbase[32 * t];
+            for (int t = 0; t < NT; ++t) {
+                bf16x8 qv;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (i + 1 < 8) {
-                const float* qrow = qbase + 2 * (i + 1) * LDQ;
-#pragma unroll
-                for (int t = 0; t < NT; ++t) qv[(i + 1) & 1][t] = qrow[32 * t];
+                for (int e = 0; e < 8; ++e) qv[e] = (__bf16)qbase[e * LDQ + 32 * t];
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qv, acc[t], 0, 0, 0);
             }
-            const float av = ar[i >> 2][i & 3];
+        } else {
+            // the panel values of k-step i+1 are read from LDS before the MFMAs of k-step i are issued
+            float qv[2][NT];
+            const float* qbase = &qs[buf][par][kh][cl];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, qv[i & 1][t], acc[t], 0, 0, 0);
+            for (int t = 0; t < NT; ++t) qv[0][t] = qbase[32 * t];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (i + 1 < 8) {
+                    const float* qrow = qbase + 2 * (i + 1) * LDQ;
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) qv[(i + 1) & 1][t] = qrow[32 * t];
+                }
+                const float av = ar[i >> 2][i & 3];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, qv[i & 1][t], acc[t], 0, 0, 0);
+            }
         }
     };
     const f4* apv = reinterpret_cast<const f4*>(ap);
     auto a_load = [&](int c, f4 (&ar)[2]) {
-        ar[0] = apv[(int64_t)c * 128];
-        ar[1] = apv[(int64_t)c * 128 + 64];
+        ar[0] = apv[(int64_t)c * APB];
+        if (!BF16) ar[1] = apv[(int64_t)c * APB + 64];
     };
 
     // Software pipeline, one chunk deep: the loads of chunk c+1 (raw panel rows and table
@@ -207,7 +226,7 @@ __global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
     }
 }
 
-template <bool ANALYSIS>
+template <bool ANALYSIS, bool BF16>
 static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     const int64_t ncols = a.ld;
     if (n_work <= 0 || ncols <= 0) return SFNO_OK;
@@ -222,7 +241,7 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
 #define LF_CASE(NT_)                                                                                 \
     case NT_: {                                                                                      \
         dim3 grid(n_work, (unsigned)((ncols + 32 * NT_ - 1) / (32 * NT_)));                          \
-        hipLaunchKernelGGL((legendre_fold_kernel<NT_, ANALYSIS>), grid, dim3(256), 0, s, a);         \
+        hipLaunchKernelGGL((legendre_fold_kernel<NT_, ANALYSIS, BF16>), grid, dim3(256), 0, s, a);   \
         break;                                                                                       \
     }
     switch (best) {
@@ -233,8 +252,9 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
-int legendre_fold_launch(bool analysis, const PgemmArgs& a, int n_work, hipStream_t s) {
-    return analysis ? launch_fold<true>(a, n_work, s) : launch_fold<false>(a, n_work, s);
+int legendre_fold_launch(bool analysis, bool bf16, const PgemmArgs& a, int n_work, hipStream_t s) {
+    if (bf16) return analysis ? launch_fold<true, true>(a, n_work, s) : launch_fold<false, true>(a, n_work, s);
+    return analysis ? launch_fold<true, false>(a, n_work, s) : launch_fold<false, false>(a, n_work, s);
 }
 
 }  // namespace sfno

@@ -67,9 +67,10 @@ struct LegendreGen {
 void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work,
                     int rb_step = PG_WAVES);
 // equator-folded Legendre streams (two per order: even and odd l+m), see tables.cpp
-void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+// bf16 = true packs 8 bf16 per lane and chunk (half the bytes; `packed` then holds 256 floats = 1 KiB per block)
+void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, bool bf16, std::vector<float>& packed,
                         std::vector<int64_t>& aoff);
-int legendre_fold_launch(bool analysis, const PgemmArgs& a, int n_work, hipStream_t s);
+int legendre_fold_launch(bool analysis, bool bf16, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
 struct FftPlan {

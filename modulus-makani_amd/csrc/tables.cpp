@@ -193,7 +193,30 @@ static void pack_blocks(float* dst, int rows, int K, G get) {
 //   analysis : rows = i, K = latitude k < ceil(nlat/2), value P*w (the equator row counted once)
 //   synthesis: rows = latitude k < ceil(nlat/2), K = i (both parities padded to the chunk count of p = 0)
 // aoff[2*m + p] = first block of that stream.
-void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, std::vector<float>& packed,
+static unsigned short bf16_rne(double v) {
+    float f = (float)v;
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// bf16 flavour of pack_blocks: block = 64 lanes x 8 bf16; lane j holds P[32 rb + (j & 31)][16 c + 8 (j >> 5) + e], e = 0..7
+template <class G>
+static void pack_blocks_bf16(unsigned short* dst, int rows, int K, G get) {
+    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
+    for (int rb = 0; rb < nrb; ++rb)
+        for (int c = 0; c < nc; ++c) {
+            unsigned short* blk = dst + ((size_t)rb * nc + c) * PG_BLOCK_FLOATS;
+            for (int j = 0; j < 64; ++j)
+                for (int e = 0; e < 8; ++e) {
+                    int row = PG_ROWS * rb + (j & 31);
+                    int k = PG_KC * c + 8 * (j >> 5) + e;
+                    blk[j * 8 + e] = (row < rows && k < K) ? bf16_rne(get(row, k)) : (unsigned short)0;
+                }
+        }
+}
+
+void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, bool bf16, std::vector<float>& packed,
                         std::vector<int64_t>& aoff) {
     const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
     const int K2 = (nlat + 1) / 2;
@@ -207,7 +230,8 @@ void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysi
             int64_t nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl_p(m, 0) + PG_KC - 1) / PG_KC;
             tot += nrb * nc;
         }
-    packed.assign((size_t)tot * PG_BLOCK_FLOATS, 0.0f);
+    const size_t blk_floats = bf16 ? PG_BLOCK_FLOATS / 2 : PG_BLOCK_FLOATS;
+    packed.assign((size_t)tot * blk_floats, 0.0f);
     float* base = packed.data();
     parallel_for(mmax, [&, base](int m) {
         int nl = lmax - m;
@@ -217,13 +241,18 @@ void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysi
         const double* r = rows.data();
         for (int p = 0; p < 2; ++p) {
             const int np = nl_p(m, p);
-            float* dst = base + (size_t)aoff[2 * m + p] * PG_BLOCK_FLOATS;
-            if (analysis) {
-                pack_blocks(dst, np, K2, [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * quad_w[k]; });
+            float* dst = base + (size_t)aoff[2 * m + p] * blk_floats;
+            // K extent of the synthesis padded to the even-parity chunk count so that both parities run the same loop
+            const int kpad = nl_p(m, 0);
+            auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * quad_w[k]; };
+            auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] : 0.0; };
+            if (bf16) {
+                unsigned short* d16 = reinterpret_cast<unsigned short*>(dst);
+                if (analysis) pack_blocks_bf16(d16, np, K2, wa);
+                else pack_blocks_bf16(d16, K2, kpad, ws);
             } else {
-                // K extent padded to the even-parity chunk count so that both parities run the same loop
-                const int kpad = nl_p(m, 0);
-                pack_blocks(dst, K2, kpad, [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] : 0.0; });
+                if (analysis) pack_blocks(dst, np, K2, wa);
+                else pack_blocks(dst, K2, kpad, ws);
             }
         }
     });

@@ -151,8 +151,11 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                  num_layers=4, repeat_layers=1, use_mlp=True, mlp_ratio=2.0, encoder_ratio=1, decoder_ratio=1, activation_function="gelu",
                  encoder_layers=1, pos_embed="none", pos_drop_rate=0.0, path_drop_rate=0.0, mlp_drop_rate=0.0,
                  normalization_layer="instance_norm", max_modes=None, hard_thresholding_fraction=1.0, big_skip=True, rank=1.0,
-                 factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0, **kwargs):
+                 factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0,
+                 spectral_compute="fp32", **kwargs):
         super().__init__()
+        # spectral_compute = "bf16" (not a Makani option) runs the Legendre and dhconv contractions on bf16 MFMA
+        self.spectral_compute = spectral_compute
         if spectral_transform != "sht":
             raise NotImplementedError("only spectral_transform='sht' runs on the HIP path")
         self.inp_shape, self.out_shape = tuple(inp_shape), tuple(out_shape)
@@ -188,6 +191,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                                            act_layer=act, norm_layer=(norm, norm), inner_skip="none", outer_skip="linear", use_mlp=use_mlp, rank=rank,
                                            factorization=factorization, separable=separable, complex_activation=complex_activation,
                                            spectral_layers=spectral_layers, bias=bias))
+            self.blocks[-1].filter.filter.compute = spectral_compute
 
         self.decoder = EncoderDecoder(encoder_layers, embed_dim, out_chans, int(decoder_ratio * embed_dim), act, gain=0.5 if big_skip else 1.0)
         if big_skip:
@@ -217,10 +221,11 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         else:
             modes_lat = int(self.h * hard_thresholding_fraction)
             modes_lon = int((self.w // 2 + 1) * hard_thresholding_fraction)
-        self.trans_down = RealSHT(*self.inp_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type).float()
-        self.itrans_up = InverseRealSHT(*self.out_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type).float()
-        self.trans = RealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type).float()
-        self.itrans = InverseRealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type).float()
+        c = self.spectral_compute
+        self.trans_down = RealSHT(*self.inp_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type, compute=c).float()
+        self.itrans_up = InverseRealSHT(*self.out_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type, compute=c).float()
+        self.trans = RealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type, compute=c).float()
+        self.itrans = InverseRealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type, compute=c).float()
         self.inp_shape_loc = (self.trans_down.nlat, self.trans_down.nlon)
         self.out_shape_loc = (self.itrans_up.nlat, self.itrans_up.nlon)
         self.h_loc, self.w_loc = self.itrans.nlat, self.itrans.nlon

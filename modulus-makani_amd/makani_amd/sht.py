@@ -69,7 +69,7 @@ class _Plan:
             check(
                 lib.sfno_sht_plan_create(
                     mod.nlat, mod.nlon, mod.lmax, mod.mmax, _lib.GRID[mod.grid], _lib.NORM[mod.norm], int(mod.csphase), directions,
-                    _lib.COMPUTE_FP32, ctypes.byref(self.handle),
+                    _lib.COMPUTE_BF16 if mod.compute == "bf16" else _lib.COMPUTE_FP32, ctypes.byref(self.handle),
                 ),
                 "sfno_sht_plan_create",
             )
@@ -91,8 +91,12 @@ def _ptr(t):
 class _SHTBase(nn.Module):
     _directions = 0
 
-    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True):
+    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, compute="fp32"):
         super().__init__()
+        # compute = "bf16": Legendre stage on bf16 MFMA (bf16 tables and inputs, fp32 accumulation); default and reference: fp32
+        if compute not in ("fp32", "bf16"):
+            raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32' or 'bf16'")
+        self.compute = compute
         self.nlat = nlat
         self.nlon = nlon
         self.grid = grid
@@ -138,7 +142,7 @@ class _SHTBase(nn.Module):
         return state
 
     def __deepcopy__(self, memo):
-        return type(self)(self.nlat, self.nlon, self.lmax, self.mmax, self.grid, self.norm, self.csphase)
+        return type(self)(self.nlat, self.nlon, self.lmax, self.mmax, self.grid, self.norm, self.csphase, self.compute)
 
 
 def _as_fp32_rows(x, tail):

@@ -147,3 +147,24 @@ def test_bf16_grid_io_equals_cast_then_transform(lib_built, nlat, nlon, lmax, mm
     y32 = isht.synthesis(s_cast, (3, 5))
     yb = isht.synthesis(s_cast, (3, 5), dtype=torch.bfloat16)
     assert yb.dtype == torch.bfloat16 and torch.equal(yb, y32.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("nlat,nlon,lmax,mmax,grid,lead", [CASES[0], CASES[3], CASES[4], CASES[8], CASES[9], (241, 480, 241, 241, "legendre-gauss", (12,))])
+def test_bf16_compute_variant(lib_built, nlat, nlon, lmax, mmax, grid, lead):
+    """Legendre stage on bf16 MFMA (bf16 tables and activations, fp32 accumulation): relative L2 <= 1e-2 vs the float64 oracle."""
+    import makani_amd as ma
+
+    print(f"case bf16 compute {nlat}x{nlon} lmax={lmax} mmax={mmax} {grid} lead={lead}", flush=True)
+    t = ShtTables(nlat, nlon, lmax, mmax, grid)
+    torch.manual_seed(8)
+    x = torch.randn(*lead, nlat, nlon)
+    got = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute="bf16")(x.cuda())
+    ref = sht_forward(x.double().numpy(), t)
+    e_fwd = rel_l2(got.cpu().numpy(), ref)
+    c = torch.randn(*lead, t.lmax, t.mmax, dtype=torch.complex64)
+    goti = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute="bf16")(c.cuda())
+    refi = sht_inverse(c.numpy().astype(np.complex128), t)
+    e_inv = rel_l2(goti.cpu().numpy(), refi)
+    print(f"   rel-L2 forward {e_fwd:.2e} inverse {e_inv:.2e}", flush=True)
+    assert e_fwd < 1e-2 and e_inv < 1e-2
+    assert e_fwd > 1e-5 or e_inv > 1e-5          # it is the reduced-precision path that ran

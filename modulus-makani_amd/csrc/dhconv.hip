@@ -13,6 +13,8 @@
 // packed complex weights into LDS once per chunk and shared by the four wavefronts as the
 // B operand.  Wavefronts whose rows lie beyond the orders present at this degree (m > l)
 // exit early, so the triangular structure costs no guarded matrix instructions.
+#include <type_traits>
+
 #include "sfno_internal.h"
 
 namespace sfno {
@@ -23,7 +25,7 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 
 // grid = (8 * ceil(L/8) * nob, row groups); VEC4: 2*I is a multiple of 4 so activation rows can be read as float4
 template <bool VEC4>
-__global__ __launch_bounds__(256) void dhconv_kernel(DhconvArgs a) {
+__global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
     constexpr int NT = DH_COLS / 32;                 // 4 column tiles per wavefront
     constexpr int LDW = DH_COLS + 32;                // pitch = 32 mod 64: the two half-waves read different banks
     __shared__ __align__(16) float ws[2][PG_KC][LDW];
@@ -42,12 +44,18 @@ __global__ __launch_bounds__(256) void dhconv_kernel(DhconvArgs a) {
     const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;      // rows (m,b) present at this degree
     const int r0 = blockIdx.y * 128;
     if (r0 >= ncols) return;
-    const bool active = r0 + 32 * wave < ncols;
+    // Row blocks of 32 present in this group; when there are only one or two (low degrees), the four
+    // wavefronts split the column tiles of those blocks instead of idling.
+    const int nrb = min(4, (ncols - r0 + 31) / 32);
+    const int ntw = nrb == 1 ? 1 : (nrb == 2 ? 2 : 4);                 // column tiles per wavefront
+    const int rb = nrb == 1 ? 0 : (nrb == 2 ? (wave >> 1) : wave);     // my row block
+    const int t0 = nrb == 1 ? wave : (nrb == 2 ? 2 * (wave & 1) : 0);  // my first column tile
+    const bool active = rb < nrb;
     const int nc = a.nc;                                           // K chunks of 16 i' (8 complex input channels)
     const int kh = lane >> 5, cl = lane & 31;
 
     // my activation row (clamped: rows past the end repeat the last one and are not stored)
-    const int n = min(r0 + 32 * wave + cl, ncols - 1);
+    const int n = min(r0 + 32 * rb + cl, ncols - 1);
     const int mm = n / a.B, bb = n - mm * a.B;
     const float* xrow = a.X + ((int64_t)mm * a.L + l) * a.ld_in + (int64_t)bb * a.I2;
     // packed weights of (l, ob): nc chunks of 8 x 64 complex, 16 bytes per thread and chunk
@@ -84,14 +92,21 @@ __global__ __launch_bounds__(256) void dhconv_kernel(DhconvArgs a) {
         const f4 r = {-w[1], w[0], -w[3], w[2]};
         *reinterpret_cast<f4*>(&ws[buf][2 * ii + 1][4 * o2]) = r;
     };
-    auto compute = [&](int buf, const f4 (&xr)[2]) {
+    // one K-chunk of MFMAs over TI column tiles starting at tile t0; no branches inside
+    auto compute_n = [&](auto ti, int buf, const f4 (&xr)[2]) {
+        constexpr int TI = decltype(ti)::value;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-            const float* wrow = &ws[buf][8 * kh + s][cl];
+            const float* wrow = &ws[buf][8 * kh + s][32 * t0 + cl];
             const float xv = xr[s >> 2][s & 3];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv, wrow[32 * t], acc[t], 0, 0, 0);
+            for (int t = 0; t < TI; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv, wrow[32 * t], acc[t], 0, 0, 0);
         }
+    };
+    auto compute = [&](int buf, const f4 (&xr)[2]) {
+        if (ntw == 4) compute_n(std::integral_constant<int, 4>(), buf, xr);
+        else if (ntw == 2) compute_n(std::integral_constant<int, 2>(), buf, xr);
+        else compute_n(std::integral_constant<int, 1>(), buf, xr);
     };
 
     // software pipeline, one chunk deep; the explicit wait at the end of each iteration keeps
@@ -123,14 +138,14 @@ __global__ __launch_bounds__(256) void dhconv_kernel(DhconvArgs a) {
     // D rows = my 32 activation rows, D cols = output columns o'
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-        const int nn = r0 + 32 * wave + 8 * (v >> 2) + 4 * kh + (v & 3);
+        const int nn = r0 + 32 * rb + 8 * (v >> 2) + 4 * kh + (v & 3);
         if (nn >= ncols) continue;
         const int m2 = nn / a.B, b2 = nn - m2 * a.B;
         float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int oc = DH_COLS * ob + 32 * t + cl;
-            if (oc < a.O2) orow[oc] = acc[t][v];
+            const int oc = DH_COLS * ob + 32 * (t0 + t) + cl;
+            if (t < ntw && oc < a.O2) orow[oc] = acc[t][v];
         }
     }
 }

@@ -35,13 +35,15 @@ __global__ __launch_bounds__(256) void coeffs_to_spectral_kernel(const float2* _
     __shared__ float2 tile[32][33];
     const int tx = threadIdx.x, ty = threadIdx.y;
     const int m0 = blockIdx.x * 32, l = blockIdx.y;
+    if (tri && m0 > l) return;          // a tile entirely above the diagonal holds nothing to move
     const int64_t r0 = (int64_t)blockIdx.z * 32;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int rr = ty + 8 * i, m = m0 + tx;
         const int64_t r = r0 + rr;
         float2 v = make_float2(0.f, 0.f);
-        if (r < rows && m < mmax) v = coeffs[(r * lmax + l) * mmax + m];
+        // orders above the degree are not moved in triangular mode: do not read them either
+        if (r < rows && m < mmax && (!tri || m <= l)) v = coeffs[(r * lmax + l) * mmax + m];
         tile[rr][tx] = v;
     }
     __syncthreads();

@@ -57,6 +57,8 @@ extern "C" {
 /* which tables a plan holds */
 #define SFNO_DIR_FORWARD 1
 #define SFNO_DIR_INVERSE 2
+#define SFNO_DIR_FORWARD_ADJOINT 4   /* tables of sfno_sht_forward_adjoint / sfno_sht_analysis_adjoint */
+#define SFNO_DIR_INVERSE_ADJOINT 8   /* tables of sfno_sht_inverse_adjoint / sfno_sht_synthesis_adjoint */
 
 /* element type of a grid-side (real field) tensor */
 #define SFNO_DTYPE_F32 0
@@ -136,6 +138,24 @@ int sfno_legendre_synthesis(const sfno_sht_plan* plan, const float* spec, float*
 /* floats in one xm buffer: mmax * nlat * ld */
 int64_t sfno_fourier_elems(const sfno_sht_plan* plan, int64_t rows);
 
+/* Vector-Jacobian products of the transforms, i.e. what autograd runs as the backward of
+ * RealSHT.forward / InverseRealSHT.forward (the reference differentiates its einsum + FFT graph;
+ * tests/test_models.py:149-157 checks that the input receives a gradient).  Gradients of complex
+ * tensors follow the PyTorch convention dL/dRe + i dL/dIm.  The plan must have been created with
+ * the matching SFNO_DIR_*_ADJOINT bit; workspace size as for the transforms themselves.
+ *   forward_adjoint : gcoeffs complex64 [rows][lmax][mmax] -> gx float32 [rows][nlat][nlon]
+ *   inverse_adjoint : gx float32 [rows][nlat][nlon] -> gcoeffs complex64 [rows][lmax][mmax]
+ *                     (zero for m > l, which the inverse transform never reads)
+ * and the same on the spectral layout, with the grid-side tensor float32 or bfloat16. */
+int sfno_sht_forward_adjoint(const sfno_sht_plan* plan, const void* gcoeffs, float* gx, int64_t rows,
+                             void* workspace, size_t workspace_bytes, void* stream);
+int sfno_sht_inverse_adjoint(const sfno_sht_plan* plan, const float* gx, void* gcoeffs, int64_t rows,
+                             void* workspace, size_t workspace_bytes, void* stream);
+int sfno_sht_analysis_adjoint(const sfno_sht_plan* plan, const float* gspec, void* gx, int x_dtype, int64_t rows,
+                              void* workspace, size_t workspace_bytes, void* stream);
+int sfno_sht_synthesis_adjoint(const sfno_sht_plan* plan, const void* gx, int x_dtype, float* gspec, int64_t rows,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* layout passes between the reference coefficient layout and the spectral layout */
 /* `triangular` != 0: only entries with m <= l are moved (to_coeffs writes zeros for
  * m > l); 0: the whole lmax x mmax rectangle is moved. */
@@ -154,6 +174,11 @@ int sfno_dhconv_weights_create(int in_channels, int out_channels, int lmax, int 
 /* (re)fill the packed stream from the current value of the parameter; enqueue only */
 int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream);
 int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w);
+/* Fills a handle created as (out_channels, in_channels, lmax) with the conjugate transpose of the
+ * parameter `weight` (complex64 [I][O][L]).  sfno_dhconv_spectral / sfno_dhconv on that handle then
+ * map the gradient of the output to the gradient of the input: gx[b,i,l,m] = sum_o gy[b,o,l,m]
+ * conj(w[i,o,l]) -- the backward of the einsum at contractions.py:130-136 with respect to `ac`. */
+int sfno_dhconv_weights_update_adjoint(sfno_dhconv_weights* w, const void* weight, void* stream);
 
 /* y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l] on spectral-layout buffers:
  * spec_in rows = batch*in_channels, spec_out rows = batch*out_channels.  With
@@ -161,6 +186,14 @@ int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w);
  * transform are zero elsewhere).  Replaces _contract_dhconv (contractions.py:130-136). */
 int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* spec_in, float* spec_out,
                          int batch, int mmax, int triangular, void* stream);
+
+/* Gradient of the contraction with respect to the weight (the einsum's backward with respect to
+ * `bc`): gweight[i,o,l] = sum_{b,m} conj(x[b,i,l,m]) gy[b,o,l,m], complex64 [I][O][L] overwritten.
+ * spec_in and gspec_out are spectral-layout buffers of batch*I and batch*O rows; `triangular` != 0
+ * sums over m <= l only. */
+int sfno_dhconv_weight_grad(int in_channels, int out_channels, int lmax, const float* spec_in,
+                            const float* gspec_out, void* gweight, int batch, int mmax, int triangular,
+                            void* stream);
 
 /* Same contraction on the reference layout: x complex64 [B][I][L][M] -> y complex64
  * [B][O][L][M] (contiguous), as the callable returned by get_contract_fun

@@ -29,11 +29,13 @@ void free_table(PgemmTable& t) {
     t = PgemmTable();
 }
 
-int build_legendre_table(const sfno_sht_plan& p, const double* theta, const double* quad_w, bool analysis, PgemmTable& t) {
-    LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, analysis ? 0 : 1, p.csphase);
+// inverse: which of the two Legendre normalisations (they differ for norm = schmidt); analysis: stream format
+int build_legendre_table(const sfno_sht_plan& p, const double* theta, const double* lat_w, const double* order_scale, bool inverse,
+                         bool analysis, PgemmTable& t) {
+    LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, inverse ? 1 : 0, p.csphase);
     std::vector<float> packed;
     std::vector<int64_t> aoff;
-    pack_legendre_fold(gen, quad_w, analysis, p.compute == SFNO_COMPUTE_BF16, packed, aoff);
+    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.compute == SFNO_COMPUTE_BF16, packed, aoff);
     // a workgroup covers two 32-row blocks of each parity
     const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
@@ -124,9 +126,12 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if (nlat < 2 || nlon < 1 || lmax < 1 || mmax < 1) return SFNO_EINVAL;
     // the forward transform keeps the first mmax of nlon/2+1 Fourier bins; the inverse zero-pads or
     // drops orders like a C2R transform, so only the forward direction bounds mmax
-    if ((directions & SFNO_DIR_FORWARD) && mmax > nlon / 2 + 1) return SFNO_EINVAL;
+    const int all_dirs = SFNO_DIR_FORWARD | SFNO_DIR_INVERSE | SFNO_DIR_FORWARD_ADJOINT | SFNO_DIR_INVERSE_ADJOINT;
+    if ((directions & (SFNO_DIR_FORWARD | SFNO_DIR_FORWARD_ADJOINT)) && mmax > nlon / 2 + 1) return SFNO_EINVAL;
+    // the adjoint of the zero-padding inverse would need Fourier bins the real FFT does not produce
+    if ((directions & SFNO_DIR_INVERSE_ADJOINT) && mmax > nlon / 2 + 1) return SFNO_EUNSUPPORTED;
     if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
-    if (!(directions & (SFNO_DIR_FORWARD | SFNO_DIR_INVERSE))) return SFNO_EINVAL;
+    if (!(directions & all_dirs) || (directions & ~all_dirs)) return SFNO_EINVAL;
     if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16) return SFNO_EUNSUPPORTED;
     sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
     if (!p) return SFNO_ENOMEM;
@@ -137,8 +142,26 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     std::vector<double> theta(nlat), w(nlat);
     int rc = quadrature(grid, nlat, theta.data(), w.data());
     if (rc == SFNO_OK) rc = fft_plan_init(p->fft, nlon);
-    if (rc == SFNO_OK && (directions & SFNO_DIR_FORWARD)) rc = build_legendre_table(*p, theta.data(), w.data(), true, p->fwd);
-    if (rc == SFNO_OK && (directions & SFNO_DIR_INVERSE)) rc = build_legendre_table(*p, theta.data(), w.data(), false, p->inv);
+    if (rc == SFNO_OK && (directions & SFNO_DIR_FORWARD))
+        rc = build_legendre_table(*p, theta.data(), w.data(), nullptr, false, true, p->fwd);
+    if (rc == SFNO_OK && (directions & SFNO_DIR_INVERSE))
+        rc = build_legendre_table(*p, theta.data(), nullptr, nullptr, true, false, p->inv);
+    // Adjoints.  The real FFT pair of this library is  F: x -> s * sum_n x_n e^{-i m phi_n}  (s = 2 pi / nlon)  and
+    // C: Y -> Re Y_0 + 2 sum_{0<m<nlon/2} Re(Y_m e^{i m phi_n}) + Re Y_{nlon/2} (-1)^n.  As real-linear maps,
+    // F^T = s * C o diag(1, 1/2, ..., 1/2, 1)  and  C^T = diag(1, 2, ..., 2, 1) o F / s, so each adjoint transform is
+    // the other FFT kernel around a Legendre stream whose orders carry those factors.
+    const bool even = nlon % 2 == 0;
+    const double s = 2.0 * 3.14159265358979323846264338327950288 / nlon;
+    if (rc == SFNO_OK && (directions & SFNO_DIR_FORWARD_ADJOINT)) {
+        std::vector<double> sc(mmax);
+        for (int m = 0; m < mmax; ++m) sc[m] = s * ((m == 0 || (even && m == nlon / 2)) ? 1.0 : 0.5);
+        rc = build_legendre_table(*p, theta.data(), w.data(), sc.data(), false, false, p->fwd_adj);
+    }
+    if (rc == SFNO_OK && (directions & SFNO_DIR_INVERSE_ADJOINT)) {
+        std::vector<double> sc(mmax);
+        for (int m = 0; m < mmax; ++m) sc[m] = ((m == 0 || (even && m == nlon / 2)) ? 1.0 : 2.0) / s;
+        rc = build_legendre_table(*p, theta.data(), nullptr, sc.data(), true, true, p->inv_adj);
+    }
     if (rc != SFNO_OK) { sfno_sht_plan_destroy(p); return rc; }
     *out = p;
     return SFNO_OK;
@@ -148,6 +171,8 @@ extern "C" int sfno_sht_plan_destroy(sfno_sht_plan* p) {
     if (!p) return SFNO_OK;
     free_table(p->fwd);
     free_table(p->inv);
+    free_table(p->fwd_adj);
+    free_table(p->inv_adj);
     fft_plan_free(p->fft);
     delete p;
     return SFNO_OK;
@@ -239,6 +264,56 @@ extern "C" int sfno_sht_inverse(const sfno_sht_plan* p, const void* coeffs, floa
     return sfno_sht_synthesis(p, w.spec, x, SFNO_DTYPE_F32, rows, workspace, workspace_bytes, stream);
 }
 
+// ---- adjoints (vector-Jacobian products of the transforms) -----------------------------------------
+
+extern "C" int sfno_sht_analysis_adjoint(const sfno_sht_plan* p, const float* gspec, void* gx, int x_dtype, int64_t rows, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    if (!p || !gspec || !gx || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_FORWARD_ADJOINT)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    const int64_t ld = sfno_spectral_ld(rows);
+    PgemmArgs a = legendre_args(p, p->fwd_adj, gspec, w.xm, ld);
+    int rc = legendre_fold_launch(false, p->compute == SFNO_COMPUTE_BF16, a, p->fwd_adj.n_work, (hipStream_t)stream);
+    if (rc != SFNO_OK) return rc;
+    return sfno_irfft(p, w.xm, gx, x_dtype, rows, stream);
+}
+
+extern "C" int sfno_sht_synthesis_adjoint(const sfno_sht_plan* p, const void* gx, int x_dtype, float* gspec, int64_t rows, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    if (!p || !gspec || !gx || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_INVERSE_ADJOINT)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = sfno_rfft(p, gx, x_dtype, w.xm, rows, stream);
+    if (rc != SFNO_OK) return rc;
+    const int64_t ld = sfno_spectral_ld(rows);
+    PgemmArgs a = legendre_args(p, p->inv_adj, w.xm, gspec, ld);
+    return legendre_fold_launch(true, p->compute == SFNO_COMPUTE_BF16, a, p->inv_adj.n_work, (hipStream_t)stream);
+}
+
+extern "C" int sfno_sht_forward_adjoint(const sfno_sht_plan* p, const void* gcoeffs, float* gx, int64_t rows, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    if (!p || !gcoeffs || !gx || !rows_ok(rows)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = coeffs_to_spectral_launch(reinterpret_cast<const float2*>(gcoeffs), w.spec, rows, p->lmax, p->mmax,
+                                       (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+    if (rc != SFNO_OK) return rc;
+    return sfno_sht_analysis_adjoint(p, w.spec, gx, SFNO_DTYPE_F32, rows, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sfno_sht_inverse_adjoint(const sfno_sht_plan* p, const float* gx, void* gcoeffs, int64_t rows, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    if (!p || !gcoeffs || !gx || !rows_ok(rows)) return SFNO_EINVAL;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = sfno_sht_synthesis_adjoint(p, gx, SFNO_DTYPE_F32, w.spec, rows, workspace, workspace_bytes, stream);
+    if (rc != SFNO_OK) return rc;
+    return spectral_to_coeffs_launch(w.spec, reinterpret_cast<float2*>(gcoeffs), rows, p->lmax, p->mmax,
+                                     (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+}
+
 extern "C" int sfno_coeffs_to_spectral(const void* coeffs, float* spec, int64_t rows, int lmax, int mmax, int triangular,
                                        void* stream) {
     if (!coeffs || !spec || !rows_ok(rows)) return SFNO_EINVAL;
@@ -281,11 +356,33 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
     return SFNO_OK;
 }
 
-extern "C" int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream) {
+static int pack_weights(sfno_dhconv_weights* w, const void* weight, int adjoint, void* stream) {
     if (!w || !weight) return SFNO_EINVAL;
     if (w->compute == SFNO_COMPUTE_BF16)
-        return dhconv_pack_bf16_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, (hipStream_t)stream);
-    return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, (hipStream_t)stream);
+        return dhconv_pack_bf16_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
+    return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
+}
+
+extern "C" int sfno_dhconv_weights_update(sfno_dhconv_weights* w, const void* weight, void* stream) {
+    return pack_weights(w, weight, 0, stream);
+}
+
+extern "C" int sfno_dhconv_weights_update_adjoint(sfno_dhconv_weights* w, const void* weight, void* stream) {
+    return pack_weights(w, weight, 1, stream);
+}
+
+extern "C" int sfno_dhconv_weight_grad(int I, int O, int L, const float* spec_in, const float* gspec_out, void* gweight, int batch,
+                                       int mmax, int triangular, void* stream) {
+    if (I < 1 || O < 1 || L < 1 || !spec_in || !gspec_out || !gweight || batch < 1 || mmax < 1) return SFNO_EINVAL;
+    DhconvWgradArgs a;
+    a.X = spec_in;
+    a.G = gspec_out;
+    a.GW = reinterpret_cast<float*>(gweight);
+    a.B = batch; a.I = I; a.O = O; a.L = L; a.M = mmax;
+    a.tri = triangular ? 1 : 0;
+    a.ld_in = (int)sfno_spectral_ld((int64_t)batch * I);
+    a.ld_out = (int)sfno_spectral_ld((int64_t)batch * O);
+    return dhconv_wgrad_launch(a, (hipStream_t)stream);
 }
 
 extern "C" int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w) {

@@ -150,9 +150,10 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
     }
 }
 
-// packed[l][ob][c][ii][o] (complex) = w[8c + ii][64 ob + o][l], zero outside the weight
+// packed[l][ob][c][ii][o] (complex) = w[8c + ii][64 ob + o][l], zero outside the weight;
+// adjoint: w is [O][I][L] and the packed element is conj(w[64 ob + o][8c + ii][l])
 __global__ __launch_bounds__(256) void dhconv_pack_kernel(const float2* __restrict__ w, float2* __restrict__ packed, int I, int O, int L,
-                                                          int nob, int nc) {
+                                                          int nob, int nc, int adjoint) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t total = (int64_t)L * nob * nc * 512;
     if (idx >= total) return;
@@ -163,16 +164,23 @@ __global__ __launch_bounds__(256) void dhconv_pack_kernel(const float2* __restri
     const int ob = (int)(rem % nob), l = (int)(rem / nob);
     const int i = 8 * c + ii, oo = 64 * ob + o;
     float2 v = make_float2(0.f, 0.f);
-    if (i < I && oo < O) v = w[((int64_t)i * O + oo) * L + l];
+    if (i < I && oo < O) {
+        if (adjoint) {
+            v = w[((int64_t)oo * I + i) * L + l];
+            v.y = -v.y;
+        } else {
+            v = w[((int64_t)i * O + oo) * L + l];
+        }
+    }
     packed[idx] = v;
 }
 
-int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, hipStream_t s) {
+int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, int adjoint, hipStream_t s) {
     const int nob = (2 * O + DH_COLS - 1) / DH_COLS, nc = (2 * I + PG_KC - 1) / PG_KC;
     const int64_t total = (int64_t)L * nob * nc * 512;
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    hipLaunchKernelGGL(dhconv_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<float2*>(packed), I, O, L, nob, nc);
+    hipLaunchKernelGGL(dhconv_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<float2*>(packed), I, O, L, nob, nc, adjoint);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
@@ -297,8 +305,9 @@ __global__ __launch_bounds__(256, 2) void dhconv_bf16_kernel(DhconvArgs a) {
 }
 
 // packed[l][ob][c][o (128)][i (16)] = bf16(re) | bf16(im) << 16 of w[16c + i][128 ob + o][l], zero outside the weight
+// (adjoint: of conj(w[128 ob + o][16c + i][l]), w being [O][I][L])
 __global__ __launch_bounds__(256) void dhconv_pack_bf16_kernel(const float2* __restrict__ w, unsigned int* __restrict__ packed, int I, int O, int L,
-                                                               int nob, int nc) {
+                                                               int nob, int nc, int adjoint) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t total = (int64_t)L * nob * nc * 2048;
     if (idx >= total) return;
@@ -310,19 +319,25 @@ __global__ __launch_bounds__(256) void dhconv_pack_bf16_kernel(const float2* __r
     const int i = 16 * c + ii, oo = 128 * ob + o;
     unsigned int v = 0;
     if (i < I && oo < O) {
-        const float2 z = w[((int64_t)i * O + oo) * L + l];
+        float2 z;
+        if (adjoint) {
+            z = w[((int64_t)oo * I + i) * L + l];
+            z.y = -z.y;
+        } else {
+            z = w[((int64_t)i * O + oo) * L + l];
+        }
         const __bf16 re = (__bf16)z.x, im = (__bf16)z.y;
         v = (unsigned int)__builtin_bit_cast(unsigned short, re) | ((unsigned int)__builtin_bit_cast(unsigned short, im) << 16);
     }
     packed[idx] = v;
 }
 
-int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, hipStream_t s) {
+int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s) {
     const int nob = (2 * O + DHB_COLS - 1) / DHB_COLS, nc = (2 * I + DHB_KC - 1) / DHB_KC;
     const int64_t total = (int64_t)L * nob * nc * 2048;
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    hipLaunchKernelGGL(dhconv_pack_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc);
+    hipLaunchKernelGGL(dhconv_pack_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc, adjoint);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

@@ -51,7 +51,17 @@ struct DhconvArgs {
 int dhconv_launch(const DhconvArgs& a, hipStream_t s);
 // bf16 MFMA variant: 256 output columns per workgroup, K chunks of 32, weights packed as complex bf16
 int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s);
-int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, hipStream_t s);
+// adjoint = 1 packs the conjugate transpose: w then has shape [O][I][L] and element (i, o) is conj(w[o][i])
+int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s);
+// gradient of the contraction with respect to its weight:
+// gw[i][o][l] = sum over rows (m, b) of conj(X[(m, l, b)][i]) * G[(m, l, b)][o]
+struct DhconvWgradArgs {
+    const float* X;                // spectral layout, rows of 2*I floats
+    const float* G;                // spectral layout, rows of 2*O floats
+    float* GW;                     // complex [I][O][L]
+    int B, I, O, L, M, tri, ld_in, ld_out;
+};
+int dhconv_wgrad_launch(const DhconvWgradArgs& a, hipStream_t s);
 
 // ---- host-side table construction (tables.cpp) -----------------------------------------
 int quadrature(int grid, int nlat, double* theta, double* w);
@@ -68,8 +78,9 @@ void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost
                     int rb_step = PG_WAVES);
 // equator-folded Legendre streams (two per order: even and odd l+m), see tables.cpp
 // bf16 = true packs 8 bf16 per lane and chunk (half the bytes; `packed` then holds 256 floats = 1 KiB per block)
-void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, bool bf16, std::vector<float>& packed,
-                        std::vector<int64_t>& aoff);
+// value = P * lat_w[k] * order_scale[m]; a null pointer stands for all ones
+void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, bool bf16,
+                        std::vector<float>& packed, std::vector<int64_t>& aoff);
 int legendre_fold_launch(bool analysis, bool bf16, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
@@ -98,13 +109,14 @@ int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, i
                               hipStream_t s);
 int spectral_to_coeffs_launch(const float* spec, float2* coeffs, int64_t rows, int lmax, int mmax, int ld, int tri,
                               hipStream_t s);
-int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, hipStream_t s);
+int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, int adjoint, hipStream_t s);
 
 }  // namespace sfno
 
 struct sfno_sht_plan {
     int nlat, nlon, lmax, mmax, grid, norm, csphase, directions, compute, device;
-    sfno::PgemmTable fwd, inv;
+    sfno::PgemmTable fwd, inv;          // analysis (forward) and synthesis (inverse) streams
+    sfno::PgemmTable fwd_adj, inv_adj;  // their adjoints: synthesis-format stream of the analysis table and vice versa
     sfno::FftPlan fft;
 };
 

@@ -190,8 +190,11 @@ static void pack_blocks(float* dst, int rows, int K, G get) {
 // (-1)^(l+m) Pbar_l^m(theta), so degrees of even and odd l+m only need the northern half of the
 // latitudes, applied to the sum resp. difference of mirrored rows.  Per order m and parity p
 // (l = m + p + 2 i) one packed stream:
-//   analysis : rows = i, K = latitude k < ceil(nlat/2), value P*w (the equator row counted once)
-//   synthesis: rows = latitude k < ceil(nlat/2), K = i (both parities padded to the chunk count of p = 0)
+//   analysis format : rows = i, K = latitude k < ceil(nlat/2) (the equator row counted once)
+//   synthesis format: rows = latitude k < ceil(nlat/2), K = i (both parities padded to the chunk count of p = 0)
+// Every value is P * lat_w[k] * order_scale[m] (either factor may be absent): the forward transform packs the
+// quadrature weights into the analysis format, the inverse packs plain P into the synthesis format, and the
+// adjoints of the two swap the formats.
 // aoff[2*m + p] = first block of that stream.
 static unsigned short bf16_rne(double v) {
     float f = (float)v;
@@ -216,8 +219,8 @@ static void pack_blocks_bf16(unsigned short* dst, int rows, int K, G get) {
         }
 }
 
-void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysis, bool bf16, std::vector<float>& packed,
-                        std::vector<int64_t>& aoff) {
+void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, bool bf16,
+                        std::vector<float>& packed, std::vector<int64_t>& aoff) {
     const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
     const int K2 = (nlat + 1) / 2;
     auto nl_p = [&](int m, int p) { return (lmax - m - p > 0) ? (lmax - m - p + 1) / 2 : 0; };
@@ -244,8 +247,10 @@ void pack_legendre_fold(const LegendreGen& g, const double* quad_w, bool analysi
             float* dst = base + (size_t)aoff[2 * m + p] * blk_floats;
             // K extent of the synthesis padded to the even-parity chunk count so that both parities run the same loop
             const int kpad = nl_p(m, 0);
-            auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * quad_w[k]; };
-            auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] : 0.0; };
+            const double sc = order_scale ? order_scale[m] : 1.0;
+            auto lw = [=](int k) { return lat_w ? lat_w[k] * sc : sc; };
+            auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * lw(k); };
+            auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] * lw(row) : 0.0; };
             if (bf16) {
                 unsigned short* d16 = reinterpret_cast<unsigned short*>(dst);
                 if (analysis) pack_blocks_bf16(d16, np, K2, wa);

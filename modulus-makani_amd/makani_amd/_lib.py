@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libsfno_spectral.so")
 
 GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2}
 NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
-DIR_FORWARD, DIR_INVERSE = 1, 2
+DIR_FORWARD, DIR_INVERSE, DIR_FORWARD_ADJOINT, DIR_INVERSE_ADJOINT = 1, 2, 4, 8
 COMPUTE_FP32, COMPUTE_BF16 = 0, 1
 DTYPE_F32, DTYPE_BF16 = 0, 1
 
@@ -46,6 +46,10 @@ def _load():
         "sfno_sht_io_dtype_supported": (i32, [vp, i32]),
         "sfno_sht_analysis": (i32, [vp, vp, i32, vp, i64, vp, sz, vp]),
         "sfno_sht_synthesis": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),
+        "sfno_sht_forward_adjoint": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_inverse_adjoint": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_analysis_adjoint": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),
+        "sfno_sht_synthesis_adjoint": (i32, [vp, vp, i32, vp, i64, vp, sz, vp]),
         "sfno_rfft": (i32, [vp, vp, i32, vp, i64, vp]),
         "sfno_irfft": (i32, [vp, vp, vp, i32, i64, vp]),
         "sfno_legendre_analysis": (i32, [vp, vp, vp, i64, vp]),
@@ -56,6 +60,8 @@ def _load():
         "sfno_dhconv_weights_create": (i32, [i32, i32, i32, i32, c.POINTER(vp)]),
         "sfno_dhconv_weights_update": (i32, [vp, vp, vp]),
         "sfno_dhconv_weights_destroy": (i32, [vp]),
+        "sfno_dhconv_weights_update_adjoint": (i32, [vp, vp, vp]),
+        "sfno_dhconv_weight_grad": (i32, [i32, i32, i32, vp, vp, vp, i32, i32, i32, vp]),
         "sfno_dhconv_spectral": (i32, [vp, vp, vp, i32, i32, i32, vp]),
         "sfno_dhconv_workspace_bytes": (sz, [vp, i32, i32]),
         "sfno_dhconv": (i32, [vp, vp, vp, i32, i32, i32, vp, sz, vp]),

@@ -7,6 +7,7 @@ import weakref
 from functools import partial
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from . import _lib
 from ._lib import lib, check
@@ -24,8 +25,10 @@ class PackedWeights:
         with torch.cuda.device(self.device):
             check(lib.sfno_dhconv_weights_create(in_channels, out_channels, lmax, COMPUTE[compute], ctypes.byref(self.handle)), "sfno_dhconv_weights_create")
 
-    def refresh(self, weight):
-        """Re-pack if the parameter changed (in-place updates bump ``_version``)."""
+    def refresh(self, weight, adjoint=False):
+        """Re-pack if the parameter changed (in-place updates bump ``_version``).
+
+        adjoint: this handle has shape (O, I, L) and is filled with the conjugate transpose of ``weight`` [I, O, L]."""
         stamp = (weight.data_ptr(), weight._version)
         if stamp != self.stamp:
             w = weight.detach()
@@ -33,7 +36,10 @@ class PackedWeights:
                 raise TypeError(f"dhconv weight must be complex64, got {w.dtype}")
             w = w.contiguous()
             s = ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
-            check(lib.sfno_dhconv_weights_update(self.handle, ctypes.c_void_p(w.data_ptr()), s), "sfno_dhconv_weights_update")
+            if adjoint:
+                check(lib.sfno_dhconv_weights_update_adjoint(self.handle, ctypes.c_void_p(w.data_ptr()), s), "sfno_dhconv_weights_update_adjoint")
+            else:
+                check(lib.sfno_dhconv_weights_update(self.handle, ctypes.c_void_p(w.data_ptr()), s), "sfno_dhconv_weights_update")
             self.stamp = stamp
         return self
 
@@ -51,24 +57,67 @@ COMPUTE = {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16}
 _cache = {}
 
 
-def packed_for(weight, compute="fp32"):
-    """Packed handle for a weight tensor, cached per tensor object and refreshed when it changes."""
+def packed_for(weight, compute="fp32", adjoint=False):
+    """Packed handle for a weight tensor (or, for the backward pass, for its conjugate transpose), cached per
+    tensor object and refreshed when it changes."""
     if weight.device.type != "cuda":
         raise RuntimeError("the dhconv kernel runs on a HIP device only")
     if compute not in COMPUTE:
         raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32' or 'bf16'")
-    key = (id(weight), compute)
+    key = (id(weight), compute, adjoint)
+    shape = (weight.shape[1], weight.shape[0], weight.shape[2]) if adjoint else tuple(weight.shape)
     hit = _cache.get(key)
     p = hit[1] if hit is not None and hit[0]() is weight else None
-    if p is None or p.device != weight.device or p.shape != tuple(weight.shape):
-        p = PackedWeights(weight.shape[0], weight.shape[1], weight.shape[2], weight.device, compute)
+    if p is None or p.device != weight.device or p.shape != shape:
+        p = PackedWeights(shape[0], shape[1], shape[2], weight.device, compute)
         _cache[key] = (weakref.ref(weight, lambda _, k=key: _cache.pop(k, None)), p)
-    return p.refresh(weight)
+    return p.refresh(weight, adjoint)
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _weight_grad(spec_in, gspec_out, shape, batch, mmax, triangular):
+    """gw[i,o,l] = sum_{b,m} conj(x[b,i,l,m]) g[b,o,l,m] from spectral-layout buffers."""
+    I, O, L = shape
+    gw = torch.empty((I, O, L), dtype=torch.complex64, device=spec_in.device)
+    check(
+        lib.sfno_dhconv_weight_grad(I, O, L, ctypes.c_void_p(spec_in.data_ptr()), ctypes.c_void_p(gspec_out.data_ptr()),
+                                    ctypes.c_void_p(gw.data_ptr()), batch, mmax, int(triangular), _stream(spec_in.device)),
+        "sfno_dhconv_weight_grad",
+    )
+    return gw
+
+
+class _DhconvSpectralFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, spec_in, weight, batch, mmax, triangular, compute):
+        ctx.save_for_backward(spec_in, weight)
+        ctx.cfg = (batch, mmax, triangular, compute)
+        return _dhconv_spectral(spec_in, weight, batch, mmax, triangular, compute, False)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        spec_in, weight = ctx.saved_tensors
+        batch, mmax, triangular, compute = ctx.cfg
+        g = g.contiguous()
+        gin = gw = None
+        if ctx.needs_input_grad[0]:
+            gin = _dhconv_spectral(g, weight, batch, mmax, triangular, compute, True)
+        if ctx.needs_input_grad[1]:
+            gw = _weight_grad(spec_in, g, tuple(weight.shape), batch, mmax, triangular)
+        return gin, gw, None, None, None, None
 
 
 def dhconv_spectral(spec_in, weight, batch, mmax, triangular=True, compute="fp32"):
     """Spectral-layout contraction: [mmax, L, ld(batch*I)] -> [mmax, L, ld(batch*O)]."""
-    pw = packed_for(weight, compute)
+    return _DhconvSpectralFn.apply(spec_in.contiguous(), weight, batch, mmax, triangular, compute)
+
+
+def _dhconv_spectral(spec_in, weight, batch, mmax, triangular, compute, adjoint):
+    pw = packed_for(weight, compute, adjoint)
     I, O, L = pw.shape
     ld_out = int(lib.sfno_spectral_ld(batch * O))
     out = torch.empty((mmax, L, ld_out), dtype=torch.float32, device=spec_in.device)
@@ -88,12 +137,46 @@ def _contract_dhconv(ac: torch.Tensor, bc: torch.Tensor, triangular: bool = Fals
         raise RuntimeError(f"dhconv: shapes {tuple(ac.shape)} and {tuple(bc.shape)} do not match 'bixy,iox->boxy'")
     if ac.dtype != torch.complex64:
         raise TypeError(f"dhconv input must be complex64, got {ac.dtype}")
-    if (ac.requires_grad or bc.requires_grad) and torch.is_grad_enabled():
-        raise NotImplementedError("backward through the HIP dhconv kernel is not implemented")
-    ac = ac.contiguous()
-    B, I, L, M = ac.shape
-    O = bc.shape[1]
-    pw = packed_for(bc, compute)
+    return _DhconvFn.apply(ac.contiguous(), bc, triangular, compute)
+
+
+def _to_spectral(c, rows, L, M, triangular):
+    spec = torch.empty((M, L, int(lib.sfno_spectral_ld(rows))), dtype=torch.float32, device=c.device)
+    check(lib.sfno_coeffs_to_spectral(ctypes.c_void_p(c.data_ptr()), ctypes.c_void_p(spec.data_ptr()), rows, L, M, int(triangular),
+                                      _stream(c.device)), "sfno_coeffs_to_spectral")
+    return spec
+
+
+class _DhconvFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ac, bc, triangular, compute):
+        ctx.save_for_backward(ac, bc)
+        ctx.cfg = (triangular, compute)
+        return _dhconv(ac, bc, triangular, compute, False)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        ac, bc = ctx.saved_tensors
+        triangular, compute = ctx.cfg
+        g = g.contiguous()
+        B, I, L, M = ac.shape
+        O = bc.shape[1]
+        gac = gbc = None
+        if ctx.needs_input_grad[0]:
+            gac = _dhconv(g, bc, triangular, compute, True)
+        if ctx.needs_input_grad[1]:
+            if g.numel() == 0:
+                gbc = torch.zeros_like(bc)
+            else:
+                gbc = _weight_grad(_to_spectral(ac, B * I, L, M, triangular), _to_spectral(g, B * O, L, M, triangular), (I, O, L), B, M, triangular)
+        return gac, gbc, None, None
+
+
+def _dhconv(ac, bc, triangular, compute, adjoint):
+    B, _, L, M = ac.shape
+    pw = packed_for(bc, compute, adjoint)
+    O = pw.shape[1]
     out = torch.empty((B, O, L, M), dtype=torch.complex64, device=ac.device)
     if out.numel() == 0:
         return out

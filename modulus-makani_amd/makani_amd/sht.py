@@ -15,6 +15,7 @@ import ctypes
 import numpy as np
 import torch
 import torch.nn as nn
+from torch.autograd.function import once_differentiable
 
 from . import _lib
 from ._lib import lib, check
@@ -90,6 +91,7 @@ def _ptr(t):
 
 class _SHTBase(nn.Module):
     _directions = 0
+    _adjoint_direction = 0
 
     def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, compute="fp32"):
         super().__init__()
@@ -118,14 +120,16 @@ class _SHTBase(nn.Module):
     def extra_repr(self):
         return f"nlat={self.nlat}, nlon={self.nlon},\n lmax={self.lmax}, mmax={self.mmax},\n grid={self.grid}, csphase={self.csphase}"
 
-    def plan(self, device):
+    def plan(self, device, adjoint=False):
+        """Device plan of the transform, or (built on the first backward pass) of its adjoint."""
         device = torch.device(device)
         if device.type != "cuda":
             raise RuntimeError("the SFNO spectral kernels run on a HIP device only; move the input to the GPU")
-        key = device.index if device.index is not None else torch.cuda.current_device()
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        key = (index, adjoint)
         p = self._plans.get(key)
         if p is None:
-            p = _Plan(self, torch.device("cuda", key), self._directions)
+            p = _Plan(self, torch.device("cuda", index), self._adjoint_direction if adjoint else self._directions)
             self._plans[key] = p
         return p
 
@@ -156,15 +160,111 @@ def _as_fp32_rows(x, tail):
     else:
         if x.dtype != torch.complex64:
             raise TypeError(f"the HIP transform computes in complex64; got {x.dtype}")
-    if x.requires_grad and torch.is_grad_enabled():
-        raise NotImplementedError("backward through the HIP spherical harmonic transforms is not implemented")
     return x.contiguous()
+
+
+def _rows(lead):
+    return int(np.prod(lead)) if len(lead) else 1
+
+
+class _ForwardFn(torch.autograd.Function):
+    """RealSHT.forward on the reference layout; backward = sfno_sht_forward_adjoint."""
+
+    @staticmethod
+    def forward(ctx, x, mod):
+        ctx.mod = mod
+        return mod._forward(x)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        mod = ctx.mod
+        g = g.contiguous()
+        lead = g.shape[:-2]
+        gx = torch.empty((*lead, mod.nlat, mod.nlon), dtype=torch.float32, device=g.device)
+        if gx.numel():
+            plan = mod.plan(g.device, adjoint=True)
+            ws, nbytes = mod.workspace(plan, _rows(lead), g.device)
+            check(lib.sfno_sht_forward_adjoint(plan.handle, _ptr(g), _ptr(gx), _rows(lead), _ptr(ws), nbytes, _stream_ptr(g.device)),
+                  "sfno_sht_forward_adjoint")
+        return gx, None
+
+
+class _AnalysisFn(torch.autograd.Function):
+    """Grid field -> spectral layout; backward = sfno_sht_analysis_adjoint in the dtype of the field."""
+
+    @staticmethod
+    def forward(ctx, x, mod, dt):
+        ctx.mod, ctx.dt, ctx.shape = mod, dt, x.shape
+        return mod._analysis(x, dt)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        mod = ctx.mod
+        g = g.contiguous()
+        rows = _rows(ctx.shape[:-2])
+        gx = torch.empty(ctx.shape, dtype=torch.bfloat16 if ctx.dt == _lib.DTYPE_BF16 else torch.float32, device=g.device)
+        plan = mod.plan(g.device, adjoint=True)
+        ws, nbytes = mod.workspace(plan, rows, g.device)
+        check(lib.sfno_sht_analysis_adjoint(plan.handle, _ptr(g), _ptr(gx), ctx.dt, rows, _ptr(ws), nbytes, _stream_ptr(g.device)),
+              "sfno_sht_analysis_adjoint")
+        return gx, None, None
+
+
+class _InverseFn(torch.autograd.Function):
+    """InverseRealSHT.forward on the reference layout; backward = sfno_sht_inverse_adjoint."""
+
+    @staticmethod
+    def forward(ctx, c, mod):
+        ctx.mod = mod
+        return mod._inverse(c)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        mod = ctx.mod
+        g = g.float().contiguous()
+        lead = g.shape[:-2]
+        gc = torch.empty((*lead, mod.lmax, mod.mmax), dtype=torch.complex64, device=g.device)
+        if gc.numel():
+            plan = mod.plan(g.device, adjoint=True)
+            ws, nbytes = mod.workspace(plan, _rows(lead), g.device)
+            check(lib.sfno_sht_inverse_adjoint(plan.handle, _ptr(g), _ptr(gc), _rows(lead), _ptr(ws), nbytes, _stream_ptr(g.device)),
+                  "sfno_sht_inverse_adjoint")
+        return gc, None
+
+
+class _SynthesisFn(torch.autograd.Function):
+    """Spectral layout -> grid field; backward = sfno_sht_synthesis_adjoint."""
+
+    @staticmethod
+    def forward(ctx, spec, mod, lead, fused):
+        ctx.mod, ctx.lead = mod, tuple(lead)
+        return mod._synthesis(spec, lead, fused)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        mod = ctx.mod
+        rows = _rows(ctx.lead)
+        plan = mod.plan(g.device, adjoint=True)
+        if g.dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16):
+            g, dt = g.contiguous(), _lib.DTYPE_BF16
+        else:
+            g, dt = g.float().contiguous(), _lib.DTYPE_F32
+        gspec = torch.empty(mod.spectral_shape(rows), dtype=torch.float32, device=g.device)
+        ws, nbytes = mod.workspace(plan, rows, g.device)
+        check(lib.sfno_sht_synthesis_adjoint(plan.handle, _ptr(g), dt, _ptr(gspec), rows, _ptr(ws), nbytes, _stream_ptr(g.device)),
+              "sfno_sht_synthesis_adjoint")
+        return gspec, None, None, None
 
 
 class RealSHT(_SHTBase):
     """Forward real spherical harmonic transform (analysis)."""
 
     _directions = _lib.DIR_FORWARD
+    _adjoint_direction = _lib.DIR_FORWARD_ADJOINT
 
     @property
     def weights(self):
@@ -175,9 +275,11 @@ class RealSHT(_SHTBase):
     def forward(self, x):
         assert x.shape[-2] == self.nlat
         assert x.shape[-1] == self.nlon
-        x = _as_fp32_rows(x, "grid")
+        return _ForwardFn.apply(_as_fp32_rows(x, "grid"), self)
+
+    def _forward(self, x):
         lead = x.shape[:-2]
-        rows = int(np.prod(lead)) if len(lead) else 1
+        rows = _rows(lead)
         out = torch.empty((*lead, self.lmax, self.mmax), dtype=torch.complex64, device=x.device)
         if rows == 0:
             return out
@@ -191,14 +293,13 @@ class RealSHT(_SHTBase):
         assert x.shape[-2] == self.nlat
         assert x.shape[-1] == self.nlon
         plan = self.plan(x.device)
-        dt = _lib.DTYPE_F32
         if x.dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16):
-            if x.requires_grad and torch.is_grad_enabled():
-                raise NotImplementedError("backward through the HIP spherical harmonic transforms is not implemented")
-            x, dt = x.contiguous(), _lib.DTYPE_BF16
-        else:
-            x = _as_fp32_rows(x, "grid")
-        rows = int(np.prod(x.shape[:-2])) if x.dim() > 2 else 1
+            return _AnalysisFn.apply(x.contiguous(), self, _lib.DTYPE_BF16)
+        return _AnalysisFn.apply(_as_fp32_rows(x, "grid"), self, _lib.DTYPE_F32)
+
+    def _analysis(self, x, dt):
+        plan = self.plan(x.device)
+        rows = _rows(x.shape[:-2])
         spec = torch.empty(self.spectral_shape(rows), dtype=torch.float32, device=x.device)
         ws, nbytes = self.workspace(plan, rows, x.device)
         check(lib.sfno_sht_analysis(plan.handle, _ptr(x), dt, _ptr(spec), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_analysis")
@@ -209,6 +310,7 @@ class InverseRealSHT(_SHTBase):
     """Inverse real spherical harmonic transform (synthesis)."""
 
     _directions = _lib.DIR_INVERSE
+    _adjoint_direction = _lib.DIR_INVERSE_ADJOINT
 
     @property
     def pct(self):
@@ -219,9 +321,11 @@ class InverseRealSHT(_SHTBase):
     def forward(self, x):
         assert x.shape[-2] == self.lmax
         assert x.shape[-1] == self.mmax
-        x = _as_fp32_rows(x, "coeffs")
+        return _InverseFn.apply(_as_fp32_rows(x, "coeffs"), self)
+
+    def _inverse(self, x):
         lead = x.shape[:-2]
-        rows = int(np.prod(lead)) if len(lead) else 1
+        rows = _rows(lead)
         out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.float32, device=x.device)
         if rows == 0:
             return out
@@ -232,12 +336,18 @@ class InverseRealSHT(_SHTBase):
 
     def synthesis(self, spec, lead, dtype=torch.float32):
         """spectral-layout float32 [mmax, lmax, ld] -> x [*lead, nlat, nlon]; dtype bfloat16 rounds inside the FFT kernel."""
-        rows = int(np.prod(lead)) if len(lead) else 1
-        assert tuple(spec.shape) == self.spectral_shape(rows) and spec.dtype == torch.float32 and spec.is_contiguous()
+        rows = _rows(lead)
+        assert tuple(spec.shape) == self.spectral_shape(rows) and spec.dtype == torch.float32
         plan = self.plan(spec.device)
-        fused = dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16)
+        fused = bool(dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16))
+        out = _SynthesisFn.apply(spec.contiguous(), self, tuple(lead), fused)
+        return out if out.dtype == dtype else out.to(dtype)
+
+    def _synthesis(self, spec, lead, fused):
+        rows = _rows(lead)
+        plan = self.plan(spec.device)
         out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.bfloat16 if fused else torch.float32, device=spec.device)
         ws, nbytes = self.workspace(plan, rows, spec.device)
         check(lib.sfno_sht_synthesis(plan.handle, _ptr(spec), _ptr(out), _lib.DTYPE_BF16 if fused else _lib.DTYPE_F32, rows, _ptr(ws), nbytes,
                                      _stream_ptr(spec.device)), "sfno_sht_synthesis")
-        return out if out.dtype == dtype else out.to(dtype)
+        return out

@@ -7,6 +7,10 @@ RealSHT / InverseRealSHT forward as called from
 makani/models/common/spectral_convolution.py:131,141, and
 makani/models/common/contractions.py:134).  It is timed by bench.py's cpu_baseline leg
 and never used by the product.
+
+With ``dtype=torch.float64`` the same op sequence is the gradient oracle of the tests: the
+reference has no hand-written backward, autograd differentiates exactly these ops
+(tests/test_models.py:149-157 of the reference checks the resulting input gradient).
 """
 import numpy as np
 import torch
@@ -15,17 +19,21 @@ from .sht import ShtTables
 
 
 class TorchRefSHT:
-    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, directions=("fwd", "inv")):
+    def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, directions=("fwd", "inv"),
+                 dtype=torch.float32):
         t = ShtTables(nlat, nlon, lmax, mmax, grid, norm, csphase)
         self.nlat, self.nlon, self.lmax, self.mmax = nlat, nlon, t.lmax, t.mmax
         self.weights = None
         self.pct = None
         if "inv" in directions:
-            self.pct = torch.from_numpy(np.ascontiguousarray(t.pct.astype(np.float32)))
+            self.pct = torch.from_numpy(np.ascontiguousarray(t.pct)).to(dtype)
         if "fwd" in directions:
-            w = t.p_analysis.astype(np.float32)
-            w *= t.quad_w[None, None, :].astype(np.float32)
-            self.weights = torch.from_numpy(np.ascontiguousarray(w))
+            if dtype == torch.float32:
+                w = t.p_analysis.astype(np.float32)
+                w *= t.quad_w[None, None, :].astype(np.float32)
+            else:
+                w = t.p_analysis * t.quad_w[None, None, :]
+            self.weights = torch.from_numpy(np.ascontiguousarray(w)).to(dtype)
 
     def forward(self, x):
         x = 2.0 * torch.pi * torch.fft.rfft(x, dim=-1, norm="forward")

@@ -265,3 +265,49 @@ def test_spectral_conv_residual_rule():
     assert res.shape == (1, 2, 25, 48) and y.shape == (1, 3, 25, 48)
     assert np.allclose(res, sht_inverse(sht_forward(x, same), up))
     assert np.allclose(y, sht_inverse(dhconv(sht_forward(x, same), w), up))
+
+
+@pytest.mark.parametrize("grid,norm,nlat,nlon,lmax,mmax", [("equiangular", "ortho", 13, 24, 11, 9), ("legendre-gauss", "schmidt", 10, 19, 10, 10)])
+def test_torch_restatement_matches_numpy_oracle_and_its_gradient_is_the_transpose(grid, norm, nlat, nlon, lmax, mmax):
+    """oracle.torch_ref in float64 is the gradient oracle of the GPU backward tests.  Pinned two ways: its values
+    equal the numpy oracle's, and its autograd gradient equals the explicit transpose of the real-linear map
+    assembled column by column from the numpy oracle (a dropped factor 2 on the non-zero orders, or a kept
+    imaginary part of the mean / Nyquist order, would show)."""
+    import torch
+    from oracle.torch_ref import TorchRefSHT
+    from oracle.sht import ShtTables, sht_forward, sht_inverse
+
+    t = ShtTables(nlat, nlon, lmax, mmax, grid, norm)
+    ref = TorchRefSHT(nlat, nlon, lmax, mmax, grid, norm, dtype=torch.float64)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((nlat, nlon))
+    c = rng.standard_normal((lmax, mmax)) + 1j * rng.standard_normal((lmax, mmax))
+    np.testing.assert_allclose(ref.forward(torch.from_numpy(x)).numpy(), sht_forward(x, t), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(ref.inverse(torch.from_numpy(c)).numpy(), sht_inverse(c, t), rtol=1e-11, atol=1e-12)
+
+    # forward: J[(l,m,re|im), (k,n)] from unit fields; gradient for cotangent g must be J^T [Re g; Im g]
+    J = np.empty((lmax, mmax, 2, nlat * nlon))
+    for j in range(nlat * nlon):
+        e = np.zeros(nlat * nlon)
+        e[j] = 1.0
+        y = sht_forward(e.reshape(nlat, nlon), t)
+        J[:, :, 0, j], J[:, :, 1, j] = y.real, y.imag
+    g = rng.standard_normal((lmax, mmax)) + 1j * rng.standard_normal((lmax, mmax))
+    xt = torch.from_numpy(x).requires_grad_(True)
+    ref.forward(xt).backward(torch.from_numpy(g))
+    want = np.einsum("lmj,lm->j", J[:, :, 0], g.real) + np.einsum("lmj,lm->j", J[:, :, 1], g.imag)
+    np.testing.assert_allclose(xt.grad.numpy().ravel(), want, rtol=1e-10, atol=1e-12)
+
+    # inverse: K[(k,n), (l,m,re|im)] from unit coefficients
+    K = np.empty((nlat * nlon, lmax, mmax, 2))
+    for l in range(lmax):
+        for m in range(mmax):
+            for p, v in enumerate((1.0, 1j)):
+                e = np.zeros((lmax, mmax), dtype=np.complex128)
+                e[l, m] = v
+                K[:, l, m, p] = sht_inverse(e, t).ravel()
+    gx = rng.standard_normal((nlat, nlon))
+    ct = torch.from_numpy(c).requires_grad_(True)
+    ref.inverse(ct).backward(torch.from_numpy(gx))
+    want = np.einsum("jlmp,j->lmp", K, gx.ravel())
+    np.testing.assert_allclose(torch.view_as_real(ct.grad).numpy(), want, rtol=1e-10, atol=1e-12)

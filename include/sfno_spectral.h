@@ -68,6 +68,10 @@ extern "C" {
 #define SFNO_COMPUTE_FP32 0      /* fp32 MFMA, fp32 tables */
 #define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs, fp32 accumulate */
 
+/* activation fused into the pointwise kernels */
+#define SFNO_ACT_NONE 0
+#define SFNO_ACT_GELU 1          /* exact (erf) GELU, torch.nn.GELU() */
+
 typedef struct sfno_sht_plan sfno_sht_plan;
 typedef struct sfno_dhconv_weights sfno_dhconv_weights;
 
@@ -202,6 +206,36 @@ int sfno_dhconv_weight_grad(int in_channels, int out_channels, int lmax, const f
 size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int mmax);
 int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y, int batch, int mmax,
                 int triangular, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- pointwise tail of the SFNO block (bf16 activations) -------------------------------- */
+
+/* 1x1 convolution on NCHW bfloat16 activations with a fused epilogue:
+ *   y[b][o][p] = act( sum_k w[o][k] x[b][k][p] + bias[o] ) + add_scale[b][o] * addend[b][o][p] + add_shift[b][o]
+ * x bf16 [B][K][P], y bf16 [B][O][P] (P = H*W, a multiple of 8); w is the weight packed by
+ * sfno_pointwise_pack_weight; bias, addend, add_scale, add_shift may be null.  fp32 accumulation, one
+ * rounding at the store.  Replaces nn.Conv2d(kernel_size=1) followed by the activation of EncoderDecoder / MLP
+ * (makani/models/common/layers.py:95-116,160-216) and, with `addend`, the "norm1(x) + outer_skip(residual)"
+ * and "decoder(x) + residual_transform(residual)" sums (makani/models/networks/sfnonet.py:258-262,636-638). */
+int sfno_pointwise_conv(const void* x, const void* w, const float* bias, void* y, int batch, int K, int O,
+                        int64_t P, int act, const void* addend, const float* add_scale, const float* add_shift,
+                        void* stream);
+
+/* Packs a 1x1 convolution weight (float32 [O][K], the nn.Conv2d parameter viewed as a matrix) into the bf16
+ * MFMA operand stream sfno_pointwise_conv reads; `packed` holds sfno_pointwise_weight_elems(O, K) bf16 values. */
+int64_t sfno_pointwise_weight_elems(int O, int K);
+int sfno_pointwise_pack_weight(const float* w, void* packed, int O, int K, void* stream);
+
+/* Instance norm as a per-(b, c) affine: scale = gamma[c] / sqrt(var + eps), shift = beta[c] - mean * scale over
+ * the P pixels of each of the `rows` = B*C rows of x (bf16), statistics in fp32 with the biased variance
+ * (nn.InstanceNorm2d(affine=True, track_running_stats=False), sfnonet.py:379-386).  gamma/beta may be null. */
+size_t sfno_instance_norm_workspace_bytes(int64_t rows, int64_t P);
+int sfno_instance_norm_coeffs(const void* x, const float* gamma, const float* beta, float* scale, float* shift,
+                              int64_t rows, int channels, int64_t P, float eps, void* workspace,
+                              size_t workspace_bytes, void* stream);
+/* y = act(scale[row] * x + shift[row]) on bf16 rows of P pixels: the norm0 -> activation step of
+ * sfnonet.py:246-251 once the coefficients above are known. */
+int sfno_scale_shift_act(const void* x, const float* scale, const float* shift, void* y, int64_t rows, int64_t P,
+                         int act, void* stream);
 
 #ifdef __cplusplus
 }

@@ -433,3 +433,53 @@ extern "C" int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y,
     if (rc != SFNO_OK) return rc;
     return sfno_spectral_to_coeffs(sout, y, (int64_t)batch * w->O, w->L, mmax, triangular, stream);
 }
+
+// ---- pointwise tail -----------------------------------------------------------------------------
+
+extern "C" int64_t sfno_pointwise_weight_elems(int O, int K) {
+    if (O < 1 || K < 1) return 0;
+    return (int64_t)pointwise_opad(O) * pointwise_kpad(K);
+}
+
+extern "C" int sfno_pointwise_pack_weight(const float* w, void* packed, int O, int K, void* stream) {
+    if (!w || !packed || O < 1 || K < 1) return SFNO_EINVAL;
+    return pointwise_pack_launch(w, reinterpret_cast<unsigned short*>(packed), O, K, (hipStream_t)stream);
+}
+
+extern "C" int sfno_pointwise_conv(const void* x, const void* w, const float* bias, void* y, int batch, int K, int O, int64_t P,
+                                   int act, const void* addend, const float* add_scale, const float* add_shift, void* stream) {
+    if (!x || !w || !y || batch < 1 || K < 1 || O < 1 || P < 1) return SFNO_EINVAL;
+    if (act != SFNO_ACT_NONE && act != SFNO_ACT_GELU) return SFNO_EINVAL;
+    PointwiseArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.X = reinterpret_cast<const unsigned short*>(x);
+    a.W = reinterpret_cast<const unsigned short*>(w);
+    a.bias = bias;
+    a.Y = reinterpret_cast<unsigned short*>(y);
+    a.addend = reinterpret_cast<const unsigned short*>(addend);
+    a.add_scale = add_scale;
+    a.add_shift = add_shift;
+    a.K = K; a.O = O; a.B = batch; a.act = act; a.P = P;
+    return pointwise_gemm_launch(a, (hipStream_t)stream);
+}
+
+extern "C" size_t sfno_instance_norm_workspace_bytes(int64_t rows, int64_t P) {
+    if (rows < 1 || P < 1) return 0;
+    return sizeof(float2) * (size_t)rows * row_stats_segments(rows, P);
+}
+
+extern "C" int sfno_instance_norm_coeffs(const void* x, const float* gamma, const float* beta, float* scale, float* shift, int64_t rows,
+                                         int channels, int64_t P, float eps, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !scale || !shift || rows < 1 || channels < 1 || P < 1) return SFNO_EINVAL;
+    if (!workspace || workspace_bytes < sfno_instance_norm_workspace_bytes(rows, P)) return SFNO_EWORKSPACE;
+    return instance_norm_coeffs_launch(reinterpret_cast<const unsigned short*>(x), gamma, beta, scale, shift, reinterpret_cast<float2*>(workspace),
+                                       rows, channels, P, eps, (hipStream_t)stream);
+}
+
+extern "C" int sfno_scale_shift_act(const void* x, const float* scale, const float* shift, void* y, int64_t rows, int64_t P, int act,
+                                    void* stream) {
+    if (!x || !scale || !shift || !y || rows < 1 || P < 1) return SFNO_EINVAL;
+    if (act != SFNO_ACT_NONE && act != SFNO_ACT_GELU) return SFNO_EINVAL;
+    return scale_shift_act_launch(reinterpret_cast<const unsigned short*>(x), scale, shift, reinterpret_cast<unsigned short*>(y), rows, P, act,
+                                  (hipStream_t)stream);
+}

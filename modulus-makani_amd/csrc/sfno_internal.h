@@ -63,6 +63,30 @@ struct DhconvWgradArgs {
 };
 int dhconv_wgrad_launch(const DhconvWgradArgs& a, hipStream_t s);
 
+// ---- pointwise tail (pointwise.hip): bf16 NCHW activations, 1x1 convolutions on bf16 MFMA ------------
+struct PointwiseArgs {
+    const unsigned short* X;       // bf16 [B][K][P]
+    const unsigned short* W;       // packed by pointwise_pack_launch
+    const float* bias;             // [O] or null
+    unsigned short* Y;             // bf16 [B][O][P]
+    const unsigned short* addend;  // bf16 [B][O][P] or null: y += add_scale[b][o] * addend + add_shift[b][o]
+    const float* add_scale;        // [B][O] or null (1)
+    const float* add_shift;        // [B][O] or null (0)
+    int K, Kpad, O, B, act;
+    int64_t P;
+    int n_oblk;                    // filled by the launcher
+    int64_t n_strips;
+};
+int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s);
+int pointwise_kpad(int K);
+int pointwise_opad(int O);
+int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, hipStream_t s);
+int row_stats_segments(int64_t rows, int64_t P);
+int instance_norm_coeffs_launch(const unsigned short* x, const float* gamma, const float* beta, float* scale, float* shift, float2* partial,
+                                int64_t rows, int channels, int64_t P, float eps, hipStream_t s);
+int scale_shift_act_launch(const unsigned short* x, const float* scale, const float* shift, unsigned short* y, int64_t rows, int64_t P, int act,
+                           hipStream_t s);
+
 // ---- host-side table construction (tables.cpp) -----------------------------------------
 int quadrature(int grid, int nlat, double* theta, double* w);
 // rows l = m..lmax-1 of order m at all latitudes: out[(l-m)*nlat + k]

@@ -15,6 +15,7 @@ NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
 DIR_FORWARD, DIR_INVERSE, DIR_FORWARD_ADJOINT, DIR_INVERSE_ADJOINT = 1, 2, 4, 8
 COMPUTE_FP32, COMPUTE_BF16 = 0, 1
 DTYPE_F32, DTYPE_BF16 = 0, 1
+ACT_NONE, ACT_GELU = 0, 1
 
 
 class SfnoError(RuntimeError):
@@ -65,6 +66,12 @@ def _load():
         "sfno_dhconv_spectral": (i32, [vp, vp, vp, i32, i32, i32, vp]),
         "sfno_dhconv_workspace_bytes": (sz, [vp, i32, i32]),
         "sfno_dhconv": (i32, [vp, vp, vp, i32, i32, i32, vp, sz, vp]),
+        "sfno_pointwise_weight_elems": (i64, [i32, i32]),
+        "sfno_pointwise_pack_weight": (i32, [vp, vp, i32, i32, vp]),
+        "sfno_pointwise_conv": (i32, [vp, vp, vp, vp, i32, i32, i32, i64, i32, vp, vp, vp, vp]),
+        "sfno_instance_norm_workspace_bytes": (sz, [i64, i64]),
+        "sfno_instance_norm_coeffs": (i32, [vp, vp, vp, vp, vp, i64, i32, i64, c.c_float, vp, sz, vp]),
+        "sfno_scale_shift_act": (i32, [vp, vp, vp, vp, i64, i64, i32, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)

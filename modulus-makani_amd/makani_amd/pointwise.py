@@ -1,0 +1,109 @@
+"""Pointwise tail of the SFNO block on the HIP kernels, for bfloat16 NCHW activations.
+
+1x1 convolutions with fused bias / exact GELU / "+ scale * addend + shift" epilogue, and
+instance norm split into its statistics (a per-(b, c) scale and shift) and their application.
+These replace the nn.Conv2d(kernel_size=1) / nn.InstanceNorm2d / nn.GELU sequences of
+makani/models/networks/sfnonet.py:246-262 and makani/models/common/layers.py:86-216 on the
+inference path under bf16 autocast; there is no backward through them.
+"""
+import ctypes
+import weakref
+
+import torch
+
+from . import _lib
+from ._lib import lib, check
+
+ACT = {None: _lib.ACT_NONE, "none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU}
+
+# id(parameter) -> (weakref, stamp, packed bf16 [O, Kpad])
+_wcache = {}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def packed_weight(weight):
+    """MFMA operand stream of a 1x1 convolution weight ([O, K, 1, 1] or [O, K]); cached per parameter and
+    rebuilt when the parameter changes."""
+    key = id(weight)
+    stamp = (weight.data_ptr(), weight._version, weight.device)
+    hit = _wcache.get(key)
+    if hit is not None and hit[0]() is weight and hit[1] == stamp:
+        return hit[2]
+    w = weight.detach().reshape(weight.shape[0], -1).float().contiguous()
+    O, K = w.shape
+    p = torch.empty(lib.sfno_pointwise_weight_elems(O, K), dtype=torch.bfloat16, device=w.device)
+    check(lib.sfno_pointwise_pack_weight(_ptr(w), _ptr(p), O, K, _stream(w.device)), "sfno_pointwise_pack_weight")
+    _wcache[key] = (weakref.ref(weight, lambda _, k=key: _wcache.pop(k, None)), stamp, p)
+    return p
+
+
+def supported(x):
+    """Whether the fused kernels take this activation tensor."""
+    return x.is_cuda and x.dim() == 4 and x.dtype == torch.bfloat16 and (x.shape[2] * x.shape[3]) % 8 == 0 and x.shape[2] * x.shape[3] >= 8
+
+
+def conv1x1(x, weight, bias=None, act=None, addend=None, add_scale=None, add_shift=None):
+    """act(conv1x1(x, weight) + bias) + add_scale * addend + add_shift  ->  bf16 [B, O, H, W]."""
+    if not supported(x):
+        raise RuntimeError("the fused pointwise kernels take contiguous bfloat16 NCHW HIP tensors with H*W a multiple of 8")
+    x = x.contiguous()
+    B, K, H, W = x.shape
+    pw = packed_weight(weight)
+    O = weight.shape[0]
+    if weight.shape[1] != K:
+        raise RuntimeError(f"conv1x1: input has {K} channels, weight expects {weight.shape[1]}")
+    y = torch.empty((B, O, H, W), dtype=torch.bfloat16, device=x.device)
+    if bias is not None:
+        bias = bias.detach().float().contiguous()
+    if addend is not None:
+        if addend.shape != y.shape or addend.dtype != torch.bfloat16:
+            raise RuntimeError("conv1x1: addend must be a bfloat16 tensor of the output's shape")
+        addend = addend.contiguous()
+        if add_scale is not None:
+            add_scale = add_scale.float().contiguous()
+            add_shift = add_shift.float().contiguous()
+            assert add_scale.numel() == B * O and add_shift.numel() == B * O
+    check(
+        lib.sfno_pointwise_conv(_ptr(x), _ptr(pw), _ptr(bias), _ptr(y), B, K, O, H * W, ACT[act], _ptr(addend), _ptr(add_scale),
+                                _ptr(add_shift), _stream(x.device)),
+        "sfno_pointwise_conv",
+    )
+    return y
+
+
+def instance_norm_coeffs(x, gamma=None, beta=None, eps=1e-5):
+    """(scale, shift) float32 [B, C] such that instance_norm(x) = scale * x + shift."""
+    if not supported(x):
+        raise RuntimeError("the fused pointwise kernels take contiguous bfloat16 NCHW HIP tensors with H*W a multiple of 8")
+    x = x.contiguous()
+    B, C, H, W = x.shape
+    rows, P = B * C, H * W
+    scale = torch.empty((B, C), dtype=torch.float32, device=x.device)
+    shift = torch.empty_like(scale)
+    nbytes = lib.sfno_instance_norm_workspace_bytes(rows, P)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    g = gamma.detach().float().contiguous() if gamma is not None else None
+    b = beta.detach().float().contiguous() if beta is not None else None
+    check(
+        lib.sfno_instance_norm_coeffs(_ptr(x), _ptr(g), _ptr(b), _ptr(scale), _ptr(shift), rows, C, P, float(eps), _ptr(ws), nbytes, _stream(x.device)),
+        "sfno_instance_norm_coeffs",
+    )
+    return scale, shift
+
+
+def scale_shift_act(x, scale, shift, act=None):
+    """act(scale[b, c] * x + shift[b, c]) -> bf16, same shape."""
+    if not supported(x):
+        raise RuntimeError("the fused pointwise kernels take contiguous bfloat16 NCHW HIP tensors with H*W a multiple of 8")
+    x = x.contiguous()
+    B, C, H, W = x.shape
+    y = torch.empty_like(x)
+    check(lib.sfno_scale_shift_act(_ptr(x), _ptr(scale), _ptr(shift), _ptr(y), B * C, H * W, ACT[act], _stream(x.device)), "sfno_scale_shift_act")
+    return y

@@ -5,8 +5,9 @@ configuration that Makani's recipes use (config/sfnonet.yaml:24-40,149-174): sam
 constructor keywords, same layer order and parameter names (``encoder.fwd.N``,
 ``blocks.i.{norm0,norm1,filter.filter,mlp.fwd.N,outer_skip}``, ``decoder.fwd.N``,
 ``residual_transform``), so a Makani state_dict loads with ``strict=True``.  The spectral
-filter runs on makani_amd.SpectralConv (HIP kernels); the pointwise parts are plain
-PyTorch modules, as in the reference.
+filter runs on makani_amd.SpectralConv (HIP kernels).  The pointwise parts are plain PyTorch
+modules, as in the reference; for inference under bf16 autocast (no gradient recorded) the
+same modules are evaluated by the fused HIP kernels of makani_amd.pointwise instead.
 """
 import math
 from functools import partial
@@ -14,10 +15,60 @@ from functools import partial
 import torch
 import torch.nn as nn
 
+from . import pointwise as pw
 from .sht import RealSHT, InverseRealSHT
 from .spectral_convolution import SpectralConv
 
 _ACTIVATIONS = {"relu": nn.ReLU, "gelu": nn.GELU, "silu": nn.SiLU}
+
+
+def _is_gelu(m):
+    return isinstance(m, nn.GELU) and getattr(m, "approximate", "none") == "none"
+
+
+def _is_conv1x1(m):
+    return isinstance(m, nn.Conv2d) and m.kernel_size == (1, 1) and m.stride == (1, 1) and m.padding == (0, 0) and m.groups == 1
+
+
+def _norm_fusable(m):
+    return isinstance(m, nn.Identity) or (isinstance(m, nn.InstanceNorm2d) and not m.track_running_stats)
+
+
+def _norm_coeffs(m, x):
+    """(scale, shift) of a fusable normalisation layer, or (None, None) for the identity."""
+    if isinstance(m, nn.Identity):
+        return None, None
+    return pw.instance_norm_coeffs(x, m.weight if m.affine else None, m.bias if m.affine else None, m.eps)
+
+
+def _fused_chain(mods):
+    """Splits a Sequential of 1x1 convolutions, GELUs and identities into (conv, act) steps; None if it holds anything else."""
+    steps = []
+    for m in mods:
+        if isinstance(m, nn.Identity):
+            continue
+        if _is_conv1x1(m):
+            steps.append([m, None])
+        elif _is_gelu(m) and steps and steps[-1][1] is None:
+            steps[-1][1] = "gelu"
+        else:
+            return None
+    return steps or None
+
+
+def _run_chain(steps, x, addend=None, add_scale=None, add_shift=None):
+    for i, (conv, act) in enumerate(steps):
+        last = i == len(steps) - 1
+        x = pw.conv1x1(x, conv.weight, conv.bias, act, addend if last else None, add_scale if last else None, add_shift if last else None)
+    return x
+
+
+def fused_pointwise_active(x):
+    """The fused kernels serve inference on bf16 activations: bf16 input or bf16 autocast, and no autograd graph."""
+    if torch.is_grad_enabled() or not x.is_cuda or x.dim() != 4:
+        return False
+    bf16 = x.dtype == torch.bfloat16 or (torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16)
+    return bf16 and (x.shape[2] * x.shape[3]) % 8 == 0
 
 
 def _pointwise(cin, cout, bias, std):
@@ -127,8 +178,31 @@ class FourierNeuralOperatorBlock(nn.Module):
         if final_activation:
             self.act_layer1 = act_layer()
 
+    def _fusable(self):
+        if not (hasattr(self, "mlp") and _fused_chain(self.mlp.fwd) and _is_gelu(self.act_layer0)):
+            return False
+        if hasattr(self, "inner_skip") or hasattr(self, "act_layer1") or not _norm_fusable(self.norm0) or not _norm_fusable(self.norm1):
+            return False
+        return hasattr(self, "outer_skip") and _is_conv1x1(self.outer_skip) and self.outer_skip.bias is None
+
+    def _forward_fused(self, x, residual):
+        """norm0 -> GELU -> MLP -> norm1 -> + outer_skip(residual) in five kernels: row statistics, scale/shift + GELU,
+        two 1x1 convolutions with bias (+ GELU) epilogues, row statistics, and the skip convolution whose epilogue adds
+        the normalised MLP output."""
+        sc, sh = _norm_coeffs(self.norm0, x)
+        if sc is None:
+            sc = torch.ones(x.shape[:2], dtype=torch.float32, device=x.device)
+            sh = torch.zeros_like(sc)
+        x = pw.scale_shift_act(x, sc, sh, "gelu")
+        x = _run_chain(_fused_chain(self.mlp.fwd), x)
+        sc, sh = _norm_coeffs(self.norm1, x)
+        return pw.conv1x1(residual, self.outer_skip.weight, None, None, x, sc, sh)
+
     def forward(self, x):
         x, residual = self.filter(x)
+        if getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 \
+                and residual.shape[2:] == x.shape[2:] and self._fusable():
+            return self._forward_fused(x.contiguous(), residual.contiguous())
         x = self.norm0(x)
         if hasattr(self, "inner_skip"):
             x = x + self.inner_skip(residual)
@@ -236,7 +310,31 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                 x = blk(x)
         return x
 
+    def _forward_fused(self, x):
+        """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""
+        enc, dec = _fused_chain(self.encoder.fwd), _fused_chain(self.decoder.fwd)
+        if self.big_skip:
+            if self.out_shape != self.inp_shape:
+                residual = self.itrans_up(self.trans_down(x.to(torch.float32)).contiguous())
+            else:
+                residual = x
+            residual = pw.conv1x1(residual.to(torch.bfloat16).contiguous(), self.residual_transform.weight)
+        x = _run_chain(enc, x.to(torch.bfloat16).contiguous())
+        x = self._forward_features(x)
+        return _run_chain(dec, x.to(torch.bfloat16).contiguous(), residual if self.big_skip else None)
+
+    def _fusable(self, x):
+        if not (getattr(self, "fused_pointwise", True) and fused_pointwise_active(x)) or hasattr(self, "pos_embed"):
+            return False
+        if not isinstance(self.pos_drop, nn.Identity) or (self.out_shape[0] * self.out_shape[1]) % 8 != 0:
+            return False
+        if self.big_skip and not (_is_conv1x1(self.residual_transform) and self.residual_transform.bias is None):
+            return False
+        return _fused_chain(self.encoder.fwd) is not None and _fused_chain(self.decoder.fwd) is not None
+
     def forward(self, x):
+        if self._fusable(x):
+            return self._forward_fused(x)
         if self.big_skip:
             if self.out_shape != self.inp_shape:
                 xtype = x.dtype

@@ -1,0 +1,116 @@
+"""GPU parity of the fused pointwise kernels (bf16 activations) against float64 PyTorch-CPU evaluation of
+the same reference ops (nn.Conv2d(k=1) + bias, nn.GELU(), nn.InstanceNorm2d) on the same bf16-rounded
+inputs.  The kernels accumulate in fp32 and round once, so the only difference is the final bf16
+rounding: relative L2 <= 3e-3 (bf16 tolerance of the path: 1e-2)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+TOL = 3e-3
+
+
+def rel_l2(a, b):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    return float(torch.linalg.norm((a - b).ravel()) / max(float(torch.linalg.norm(b.ravel())), 1e-300))
+
+
+CONV_CASES = [
+    # B, K, O, H, W, bias, act, addend, affine
+    (2, 384, 768, 16, 24, True, "gelu", False, False),     # MLP fc1
+    (1, 768, 384, 16, 24, True, None, False, False),       # MLP fc2
+    (2, 384, 384, 13, 8, False, None, True, True),         # outer skip + norm1(y); strip shorter than a tile
+    (1, 73, 384, 20, 36, True, "gelu", False, False),      # encoder fc1: K padded 73 -> 128
+    (1, 384, 73, 20, 36, False, None, True, False),        # decoder fc2 + big skip (O < 96: four wavefronts along pixels)
+    (3, 73, 73, 9, 8, False, None, False, False),
+    (1, 100, 200, 11, 24, True, "gelu", True, True),       # nothing a multiple of the tile sizes
+    (1, 8, 5, 721, 1440, True, None, False, False),        # full-resolution grid, tiny channels
+]
+
+
+@pytest.mark.parametrize("B,K,O,H,W,bias,act,addend,affine", CONV_CASES)
+def test_conv1x1(lib_built, B, K, O, H, W, bias, act, addend, affine):
+    from makani_amd import pointwise as pw
+
+    print(f"case conv1x1 B={B} K={K} O={O} {H}x{W} bias={bias} act={act} addend={addend} affine={affine}", flush=True)
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(B, K, H, W, generator=g).bfloat16()
+    w = (torch.randn(O, K, 1, 1, generator=g) / np.sqrt(K))
+    bvec = torch.randn(O, generator=g) if bias else None
+    r = torch.randn(B, O, H, W, generator=g).bfloat16() if addend else None
+    sc = torch.randn(B, O, generator=g) if affine else None
+    sh = torch.randn(B, O, generator=g) if affine else None
+
+    ref = F.conv2d(x.double(), w.bfloat16().double(), bvec.double() if bias else None)
+    if act == "gelu":
+        ref = F.gelu(ref)
+    if addend:
+        ref = ref + (r.double() * sc.double()[:, :, None, None] + sh.double()[:, :, None, None] if affine else r.double())
+
+    wg = w.cuda()
+    got = pw.conv1x1(x.cuda(), wg, bvec.cuda() if bias else None, act, r.cuda() if addend else None,
+                     sc.cuda() if affine else None, sh.cuda() if affine else None)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and got.shape == ref.shape
+    assert rel_l2(got, ref) < TOL
+    # the error of every element is bf16 rounding of the float64 value (plus fp32 accumulation noise)
+    err = (got.cpu().double() - ref).abs()
+    assert float((err - (ref.abs() * 2.0**-8 + 1e-3)).max()) <= 0.0
+
+
+def test_weight_repack_on_update(lib_built):
+    from makani_amd import pointwise as pw
+
+    x = torch.randn(1, 16, 4, 8).bfloat16().cuda()
+    w = torch.randn(8, 16, 1, 1).cuda()
+    y0 = pw.conv1x1(x, w)
+    w.mul_(2.0)
+    y1 = pw.conv1x1(x, w)
+    assert rel_l2(y1, 2.0 * y0.float()) < TOL
+
+
+@pytest.mark.parametrize("B,C,H,W", [(2, 6, 16, 24), (1, 384, 24, 48), (1, 3, 721, 1440)])
+def test_instance_norm_coeffs(lib_built, B, C, H, W):
+    from makani_amd import pointwise as pw
+
+    print(f"case instnorm B={B} C={C} {H}x{W}", flush=True)
+    g = torch.Generator().manual_seed(22)
+    # a mean several times the spread is the hard case for the variance; the scale/shift form itself loses
+    # about eps_fp32 * |mean| / sigma of relative accuracy, so the spread is kept away from zero
+    x = (torch.randn(B, C, H, W, generator=g) * (0.5 + torch.rand(B, C, 1, 1, generator=g)) + 5.0 * torch.randn(B, C, 1, 1, generator=g)).bfloat16()
+    gamma, beta = torch.randn(C, generator=g), torch.randn(C, generator=g)
+    ref = F.instance_norm(x.double(), weight=gamma.double(), bias=beta.double(), eps=1e-6)
+    scale, shift = pw.instance_norm_coeffs(x.cuda(), gamma.cuda(), beta.cuda(), eps=1e-6)
+    got = scale.cpu().double()[:, :, None, None] * x.double() + shift.cpu().double()[:, :, None, None]
+    assert rel_l2(got, ref) < 1e-5
+    y = pw.scale_shift_act(x.cuda(), scale, shift, None)
+    torch.cuda.synchronize()
+    assert rel_l2(y, ref) < TOL
+    y = pw.scale_shift_act(x.cuda(), scale, shift, "gelu")
+    assert rel_l2(y, F.gelu(ref)) < TOL
+
+
+def test_gelu_matches_erf_form(lib_built):
+    """The kernel's GELU against torch's exact (erf) GELU over [-12, 12]: equal after bf16 rounding up to one ulp
+    (2^-8 relative) plus 1e-8 absolute, which only matters in the far negative tail where |gelu| < 1e-6."""
+    from makani_amd import pointwise as pw
+
+    x = torch.linspace(-12.0, 12.0, 8 * 4096).bfloat16().reshape(1, 1, 8, 4096).cuda()
+    one = torch.ones(1, 1, device="cuda")
+    y = pw.scale_shift_act(x, one, torch.zeros_like(one), "gelu").float().cpu()
+    ref = F.gelu(x.cpu().double())
+    err = (y.double() - ref).abs()
+    assert float((err - ref.abs() * 2.0**-8).max()) <= 1e-8
+
+
+def test_unsupported_inputs_raise(lib_built):
+    from makani_amd import pointwise as pw
+
+    w = torch.randn(4, 4, 1, 1).cuda()
+    with pytest.raises(RuntimeError):
+        pw.conv1x1(torch.randn(1, 4, 4, 8).cuda(), w)                 # float32 activations
+    with pytest.raises(RuntimeError):
+        pw.conv1x1(torch.randn(1, 4, 3, 5).bfloat16().cuda(), w)      # H*W not a multiple of 8
+    with pytest.raises(RuntimeError):
+        pw.conv1x1(torch.randn(1, 4, 4, 8).bfloat16(), w.cpu())       # CPU tensor

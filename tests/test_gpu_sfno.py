@@ -106,3 +106,42 @@ def test_rollout_feeds_output_back(lib_built):
             g = net(g)
             r = oracle.forward(net.state_dict(), r).float()
     assert rel_l2(g.cpu().double().numpy(), r.double().numpy()) < 1e-4
+
+
+def test_fused_pointwise_tail_matches_module_path(lib_built):
+    """Under bf16 autocast without autograd the 1x1 convolutions, instance norms and GELUs run on the fused HIP
+    kernels.  Same network, fused against the PyTorch module path (the reference's execution).  Both round every
+    layer's output to bf16, at different places, so they are compared through the float64 oracle model: the fused
+    run (fp32 accumulation, one rounding per layer) must be no further from it than the module path is, and the
+    two runs must agree within the sum of those distances."""
+    case = dict(inp_shape=(91, 180), out_shape=(91, 180), inp_chans=5, out_chans=5, scale_factor=3, embed_dim=48, num_layers=3)
+    print(f"case sfno fused pointwise {case}", flush=True)
+    net = build(**case).cuda().eval()
+    # non-trivial affine parameters and biases, which the initialisation leaves at one and zero
+    g = torch.Generator().manual_seed(9)
+    with torch.no_grad():
+        for n, p in net.named_parameters():
+            if "norm" in n or n.endswith(".bias"):
+                p.add_(0.3 * torch.randn(p.shape, generator=g).to(p.device))
+    x = torch.randn(2, 5, 91, 180, generator=torch.Generator().manual_seed(5))
+
+    def run(fused):
+        net.fused_pointwise = fused
+        for b in net.blocks:
+            b.fused_pointwise = fused
+        with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+            return net(x.cuda())
+
+    y_fused, y_mod = run(True), run(False)
+    torch.cuda.synchronize()
+    assert y_fused.dtype == torch.bfloat16 and y_fused.shape == y_mod.shape
+    ref64 = SfnoOracle((91, 180), (91, 180), 3, 3).forward(net.state_dict(), x).numpy()
+    e_fused = rel_l2(y_fused.float().cpu().double().numpy(), ref64)
+    e_mod = rel_l2(y_mod.float().cpu().double().numpy(), ref64)
+    print(f"fused {e_fused:.3e}  module path {e_mod:.3e}", flush=True)
+    assert e_fused < 2e-2 and e_fused < 1.2 * e_mod
+    assert rel_l2(y_fused.float().cpu().numpy(), y_mod.float().cpu().numpy()) < e_fused + e_mod
+    # with autograd recording, the module path runs (the fused kernels have no backward)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y_grad = net(x.cuda().requires_grad_(True))
+    assert y_grad.requires_grad

@@ -14,7 +14,7 @@
 // A wavefront owns 96 output rows x 64 pixels (3 x 2 tiles, 96 accumulator registers), eight wavefronts
 // make a workgroup, two per SIMD.  Weights come from global memory (L2 resident) as A fragments, packed so
 // that a fragment is 1 KiB of consecutive memory; the activation chunk (16 k rows) is shared through a
-// double-buffered LDS stage; both operand streams are prefetched several chunks ahead in registers: the
+// triple-buffered LDS stage; both operand streams are prefetched several chunks ahead in registers: the
 // loads in flight, not the arithmetic, bound this kernel (the activations stream from HBM).
 #include "sfno_internal.h"
 
@@ -30,7 +30,8 @@ constexpr int PW_MT = 3;          // 32-row tiles per wavefront
 constexpr int PW_NT = 2;          // pixels per lane = N tiles per wavefront
 constexpr int PW_ROWS = 32 * PW_MT;
 constexpr int PW_PX = 32 * PW_NT; // pixels per wavefront
-constexpr int PW_KC = 16;         // k rows per chunk (one MFMA K step)
+constexpr int PW_KC = 16;         // k rows per MFMA K step
+constexpr int PW_KS = 2;          // MFMA K steps per chunk (one LDS stage, one barrier)
 constexpr int PW_KALIGN = 128;    // K is padded to whole unrolled loop bodies (PW_KC * prefetch distance)
 constexpr int PW_THREADS = 512;
 
@@ -58,10 +59,13 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
     constexpr int WN = 8 / WM;
     constexpr int WPX = WN * PW_PX;               // pixels per workgroup
     constexpr int PITCH = WPX * 2 + 16;           // bytes per LDS row
-    constexpr int D = (WM == 4) ? 8 : 4;          // prefetch distance in chunks
-    constexpr int XW = (WM == 4) ? 1 : 4;         // 8-byte words of the activation chunk per thread
-    static_assert(PW_KALIGN % (PW_KC * D) == 0, "loop body divides the padded K");
-    __shared__ __align__(16) unsigned char lds[2][PW_KC * PITCH];
+    constexpr int CK = PW_KC * PW_KS;             // k rows per chunk = per loop step
+    constexpr int STAGE = CK * PITCH;
+    constexpr int D = (WM == 4) ? 4 : 2;          // prefetch distance in chunks
+    constexpr int XW = (WM == 4) ? 1 : 4;         // 16-byte pieces of the activation chunk per thread
+    static_assert(PW_KALIGN % (CK * D) == 0, "loop body divides the padded K");
+    static_assert(CK * WPX * 2 == XW * 16 * PW_THREADS, "chunk split evenly over the threads");
+    __shared__ __align__(16) unsigned char lds[3 * STAGE];
 
     const int xcd = blockIdx.x & 7, qid = blockIdx.x >> 3;
     const int ob = qid % a.n_oblk;
@@ -77,71 +81,47 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
     const int pxw = (WM == 4 ? (wave & 1) : wave) * PW_PX;                // wavefront's pixel offset inside the stage
 
     const unsigned short* __restrict__ X = a.X + (int64_t)b * a.K * a.P;
-    // this thread's share of an activation chunk (16 k rows x WPX pixels): WM = 4: one 8-byte piece (4 pixels),
-    // WM = 1: two 16-byte pieces (8 pixels each)
-    int xr[2];
-    int64_t xoff[2];
-    int loff[2];
-    if constexpr (WM == 4) {
-        xr[0] = tid >> 5;
-        const int c4 = tid & 31;
-        xoff[0] = min(pw0 + 4 * c4, a.P - 4);                             // past the end: valid pixels, masked at the store
-        loff[0] = xr[0] * PITCH + 8 * c4;
-        xr[1] = 0; xoff[1] = 0; loff[1] = 0;
-    } else {
+    // this thread's 16-byte pieces (8 pixels of one k row) of an activation chunk of CK rows x WPX pixels
+    int xr[XW], loff[XW];
+    int64_t xoff[XW];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int e = tid + PW_THREADS * u;
-            xr[u] = e >> 6;
-            const int c8 = e & 63;
-            xoff[u] = min(pw0 + 8 * c8, a.P - 8);
-            loff[u] = xr[u] * PITCH + 16 * c8;
-        }
+    for (int u = 0; u < XW; ++u) {
+        const int e = tid + PW_THREADS * u;
+        xr[u] = e / (WPX / 8);
+        const int c8 = e - xr[u] * (WPX / 8);
+        xoff[u] = min(pw0 + 8 * c8, a.P - 8);                             // past the end: valid pixels, masked at the store
+        loff[u] = xr[u] * PITCH + 16 * c8;
     }
     // weight fragments: packed blocks of 32 rows x 16 k, 16 bytes per lane (see pointwise_pack_kernel)
-    const int nc = a.Kpad / PW_KC;
+    const int nc16 = a.Kpad / PW_KC;
     const unsigned short* wrow[PW_MT];
 #pragma unroll
-    for (int mt = 0; mt < PW_MT; ++mt) wrow[mt] = a.W + ((int64_t)(o0 / 32 + mt) * nc * 64 + lane) * 8;
+    for (int mt = 0; mt < PW_MT; ++mt) wrow[mt] = a.W + ((int64_t)(o0 / 32 + mt) * nc16 * 64 + lane) * 8;
 
-    // Kpad is a multiple of PW_KC * D: the unrolled loop below has no conditional steps, which keeps the
+    // Kpad is a multiple of CK * D: the unrolled loop below has no conditional steps, which keeps the
     // compiler's count of loads in flight exact (a skipped step would make it wait for nearly all of them)
-    const int nchunks = nc;
-    u32x4 araw[D][PW_MT];
-    u32x2 xraw[D][XW];
+    const int nchunks = a.Kpad / CK;
+    u32x4 araw[D][PW_KS][PW_MT];
+    u32x4 xraw[D][XW];
 
-    auto load_a = [&](int c, u32x4 (&dst)[PW_MT]) {
+    auto load_a = [&](int c, u32x4 (&dst)[PW_KS][PW_MT]) {
         const int cc = min(c, nchunks - 1);
 #pragma unroll
-        for (int mt = 0; mt < PW_MT; ++mt) dst[mt] = *reinterpret_cast<const u32x4*>(wrow[mt] + cc * 512);
+        for (int ks = 0; ks < PW_KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < PW_MT; ++mt) dst[ks][mt] = *reinterpret_cast<const u32x4*>(wrow[mt] + (cc * PW_KS + ks) * 512);
     };
-    auto load_x = [&](int c, u32x2 (&dst)[XW]) {
+    auto load_x = [&](int c, u32x4 (&dst)[XW]) {
         const int cc = min(c, nchunks - 1);
-        if constexpr (WM == 4) {
-            const int k = min(cc * PW_KC + xr[0], a.K - 1);               // rows past K meet zero weights
-            dst[0] = *reinterpret_cast<const u32x2*>(X + (int64_t)k * a.P + xoff[0]);
-        } else {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int k = min(cc * PW_KC + xr[u], a.K - 1);
-                const u32x4 v = *reinterpret_cast<const u32x4*>(X + (int64_t)k * a.P + xoff[u]);
-                dst[2 * u][0] = v[0]; dst[2 * u][1] = v[1];
-                dst[2 * u + 1][0] = v[2]; dst[2 * u + 1][1] = v[3];
-            }
+        for (int u = 0; u < XW; ++u) {
+            const int k = min(cc * CK + xr[u], a.K - 1);                  // rows past K meet zero weights
+            dst[u] = *reinterpret_cast<const u32x4*>(X + (int64_t)k * a.P + xoff[u]);
         }
     };
-    auto store_x = [&](int stage, const u32x2 (&src)[XW]) {
-        if constexpr (WM == 4) {
-            *reinterpret_cast<u32x2*>(&lds[stage][loff[0]]) = src[0];
-        } else {
+    auto store_x = [&](int stage, const u32x4 (&src)[XW]) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                u32x4 v;
-                v[0] = src[2 * u][0]; v[1] = src[2 * u][1];
-                v[2] = src[2 * u + 1][0]; v[3] = src[2 * u + 1][1];
-                *reinterpret_cast<u32x4*>(&lds[stage][loff[u]]) = v;
-            }
-        }
+        for (int u = 0; u < XW; ++u) *reinterpret_cast<u32x4*>(&lds[stage * STAGE + loff[u]]) = src[u];
     };
 
     f32x16 acc[PW_MT][PW_NT];
@@ -152,47 +132,59 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
 
-    // prologue: chunk 0 into LDS, chunks 1..D of the activations and 0..D-1 of the weights in flight
+    // prologue: chunks 0 and 1 into LDS, chunks 2..D+1 of the activations and 0..D-1 of the weights in flight
     {
-        u32x2 x0[XW];
+        u32x4 x0[XW], x1[XW];
         load_x(0, x0);
+        load_x(1, x1);
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            load_x(d + 1, xraw[(d + 1) % D]);
+            load_x(d + 2, xraw[(d + 2) % D]);
             load_a(d, araw[d]);
         }
         store_x(0, x0);
+        store_x(1, x1);
     }
     __syncthreads();
 
-    const unsigned char* fragbase = &lds[0][0] + (8 * ko) * PITCH + (pxw + 2 * q) * 2;
+    // B fragments: lane = pixel pair q, k rows 8 ko .. 8 ko + 7 of a 16-row sub-step.  The raw words of the next
+    // sub-step are read while the MFMAs of the current one run (hence three stages: chunk c + 1 is read during chunk c).
+    const unsigned char* fragbase = &lds[0] + (8 * ko) * PITCH + (pxw + 2 * q) * 2;
+    unsigned int rw[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const unsigned int*>(fragbase + r * PITCH);
+    int s0 = 0;                                    // stage of chunk c
     for (int c0 = 0; c0 < nchunks; c0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
             const int c = c0 + u;
-            // B fragments of chunk c from LDS stage c & 1: lane = pixel pair q, k rows 8 ko .. 8 ko + 7
-            const unsigned char* fb = fragbase + (c & 1) * (PW_KC * PITCH);
-            unsigned int rw[8];
+            const int s1 = (s0 == 2) ? 0 : s0 + 1; // stage of chunk c + 1
+            const int s2 = (s1 == 2) ? 0 : s1 + 1; // stage of chunk c + 2
 #pragma unroll
-            for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const unsigned int*>(fb + r * PITCH);
-            u32x4 bf[PW_NT];
+            for (int ks = 0; ks < PW_KS; ++ks) {
+                u32x4 bf[PW_NT];
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                bf[0][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x05040100u);
-                bf[1][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x07060302u);
+                for (int h = 0; h < 4; ++h) {
+                    bf[0][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x05040100u);
+                    bf[1][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x07060302u);
+                }
+                const unsigned char* fb = (ks + 1 < PW_KS) ? fragbase + s0 * STAGE + (ks + 1) * PW_KC * PITCH : fragbase + s1 * STAGE;
+#pragma unroll
+                for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const unsigned int*>(fb + r * PITCH);
+#pragma unroll
+                for (int mt = 0; mt < PW_MT; ++mt) {
+                    const bf16x8 av = __builtin_bit_cast(bf16x8, araw[u][ks][mt]);
+#pragma unroll
+                    for (int t = 0; t < PW_NT; ++t)
+                        acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int mt = 0; mt < PW_MT; ++mt) {
-                const bf16x8 av = __builtin_bit_cast(bf16x8, araw[u][mt]);
-#pragma unroll
-                for (int t = 0; t < PW_NT; ++t)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
-            }
-            // hand chunk c + 1 to the other stage, then refill the two register slots
-            store_x((c + 1) & 1, xraw[(u + 1) % D]);
-            load_x(c + 1 + D, xraw[(u + 1) % D]);
+            // hand chunk c + 2 to its stage, then refill the two register slots
+            store_x(s2, xraw[(u + 2) % D]);
+            load_x(c + 2 + D, xraw[(u + 2) % D]);
             load_a(c + D, araw[u]);
             __syncthreads();
+            s0 = s1;
         }
     }
 

@@ -201,7 +201,7 @@ def bench_sht_pair(args):
             "nlat": nlat, "nlon": nlon, "lmax": lmax, "mmax": mmax, "batch": 1, "channels": C,
         },
         "roofline": {
-            "kernel": f"pgemm_kernel ({dom})",
+            "kernel": f"legendre_fold_kernel ({dom})",
             "bound": "mfma",
             "achieved": achieved,
             "peak": PEAK_FP32_MFMA_TFLOPS,

@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--compute", default="fp32", choices=["fp32", "bf16"],
                     help="arithmetic of the Legendre and dhconv contractions: fp32 MFMA (reference precision) or bf16 MFMA inputs with fp32 accumulation")
+    ap.add_argument("--rollout-steps", type=int, default=12, help="autoregressive steps timed by --workload rollout")
+    ap.add_argument("--rollout-warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--yardstick", action="store_true",
                     help="also run one plain 256 MiB elementwise copy (mul by 1): the known-size reference for FETCH_SIZE/WRITE_SIZE runs")
@@ -328,10 +330,10 @@ def bench_rollout(args):
     torch.cuda.set_device(dev)
     net = build_sfno8l(dev, args.compute)
     x0 = torch.randn(4, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
-    nsteps = 12
+    nsteps = args.rollout_steps
     with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
         x = x0
-        for _ in range(2):
+        for _ in range(args.rollout_warmup):
             x = net(x).float()
         torch.cuda.synchronize()
         x = x0
@@ -341,12 +343,15 @@ def bench_rollout(args):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     finite = bool(torch.isfinite(x).all())
+    # HBM bytes per rollout step, all kernels, from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
+    traffic = read_traffic("rollout_step_batch4") if args.compute == "fp32" else None
     return {
-        "metric": "SFNO-L8 rollout ms/step", "value": dt / nsteps * 1e3, "unit": "ms/step", "n_gpus": 1, "steps": nsteps, "warmup": 2,
+        "metric": "SFNO-L8 rollout ms/step", "value": dt / nsteps * 1e3, "unit": "ms/step", "n_gpus": 1, "steps": nsteps, "warmup": args.rollout_warmup,
         "ms_per_step": dt / nsteps * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 pointwise / f32 spectral", "data": "synthetic",
         "config": {"workload": "configs[4]: SFNO-8L, batch 4, 12-step autoregressive rollout, bf16 autocast"},
         "ms_per_sample_step": dt / nsteps / 4 * 1e3, "finite": finite,
+        "hbm_traffic_bytes_per_step": traffic, "hbm_traffic_bytes_total": traffic * nsteps if traffic else None,
     }
 
 

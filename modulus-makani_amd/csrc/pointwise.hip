@@ -11,11 +11,11 @@
 // (4 bytes) of 8 consecutive k rows and regroups them with byte permutes into two B fragments, one
 // per pixel of its pair; MFMA column q of N-tile t then stands for pixel 2q + t, so every lane ends up
 // with 2 consecutive pixels of each output row and stores them as one 4-byte piece.
-// A wavefront owns 96 output rows x 64 pixels (3 x 2 tiles, 96 accumulator registers), eight wavefronts
-// make a workgroup, two per SIMD.  Weights come from global memory (L2 resident) as A fragments, packed so
-// that a fragment is 1 KiB of consecutive memory; the activation chunk (16 k rows) is shared through a
-// triple-buffered LDS stage; both operand streams are prefetched several chunks ahead in registers: the
-// loads in flight, not the arithmetic, bound this kernel (the activations stream from HBM).
+// Two kernels.  Convolutions with at most 96 output channels (pw_gemm_kernel): a wavefront owns 96 rows x 64
+// pixels, eight wavefronts side by side along the pixels; weights come from global memory (L2 resident) as A
+// fragments, packed so that a fragment is 1 KiB of consecutive memory, activations through a triple-buffered LDS
+// stage, both prefetched in registers.  All others (pw_gemm_dma_kernel, further down): 384 rows x 256 pixels per
+// workgroup with both operand streams loaded straight into LDS.
 #include "sfno_internal.h"
 
 namespace sfno {
@@ -27,13 +27,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int PW_MT = 3;          // 32-row tiles per wavefront
-constexpr int PW_NT = 2;          // pixels per lane = N tiles per wavefront
 constexpr int PW_ROWS = 32 * PW_MT;
-constexpr int PW_PX = 32 * PW_NT; // pixels per wavefront
 constexpr int PW_KC = 16;         // k rows per MFMA K step
 constexpr int PW_KS = 2;          // MFMA K steps per chunk (one LDS stage, one barrier)
 constexpr int PW_KALIGN = 128;    // K is padded to whole unrolled loop bodies (PW_KC * prefetch distance)
-constexpr int PW_THREADS = 512;
 
 __device__ __forceinline__ float bf16_to_f(unsigned short h) { return __uint_as_float((unsigned int)h << 16); }
 __device__ __forceinline__ unsigned short f_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
@@ -54,15 +51,20 @@ __device__ __forceinline__ float gelu(float x) {
 
 // WM = wavefronts along the output rows: 4 (x 2 along pixels: 384 rows x 128 pixels per workgroup) or
 // 1 (x 8 along pixels: 96 rows x 512 pixels, for convolutions with few output channels)
-template <int WM>
-__global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
-    constexpr int WN = 8 / WM;
+// NT = pixels per lane = N tiles per wavefront: 2 (eight wavefronts of 96 x 64, two per SIMD) or 4 (four wavefronts of
+// 96 x 128, one per SIMD, half the weight-fragment traffic per MFMA)
+template <int WM, int NT>
+__global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseArgs a) {
+    constexpr int NW = (NT == 2) ? 8 : 4;         // wavefronts per workgroup
+    constexpr int PW_THREADS = 64 * NW;
+    constexpr int PW_PX = 32 * NT;                // pixels per wavefront
+    constexpr int WN = NW / WM;
     constexpr int WPX = WN * PW_PX;               // pixels per workgroup
     constexpr int PITCH = WPX * 2 + 16;           // bytes per LDS row
     constexpr int CK = PW_KC * PW_KS;             // k rows per chunk = per loop step
     constexpr int STAGE = CK * PITCH;
     constexpr int D = (WM == 4) ? 4 : 2;          // prefetch distance in chunks
-    constexpr int XW = (WM == 4) ? 1 : 4;         // 16-byte pieces of the activation chunk per thread
+    constexpr int XW = CK * WPX * 2 / (16 * PW_THREADS);   // 16-byte pieces of the activation chunk per thread
     static_assert(PW_KALIGN % (CK * D) == 0, "loop body divides the padded K");
     static_assert(CK * WPX * 2 == XW * 16 * PW_THREADS, "chunk split evenly over the threads");
     __shared__ __align__(16) unsigned char lds[3 * STAGE];
@@ -77,8 +79,8 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = lane & 31, ko = lane >> 5;
-    const int o0 = ob * (PW_ROWS * WM) + (WM == 4 ? (wave >> 1) * PW_ROWS : 0);
-    const int pxw = (WM == 4 ? (wave & 1) : wave) * PW_PX;                // wavefront's pixel offset inside the stage
+    const int o0 = ob * (PW_ROWS * WM) + (wave / WN) * PW_ROWS;
+    const int pxw = (wave % WN) * PW_PX;                                  // wavefront's pixel offset inside the stage
 
     const unsigned short* __restrict__ X = a.X + (int64_t)b * a.K * a.P;
     // this thread's 16-byte pieces (8 pixels of one k row) of an activation chunk of CK rows x WPX pixels
@@ -124,11 +126,11 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
         for (int u = 0; u < XW; ++u) *reinterpret_cast<u32x4*>(&lds[stage * STAGE + loff[u]]) = src[u];
     };
 
-    f32x16 acc[PW_MT][PW_NT];
+    f32x16 acc[PW_MT][NT];
 #pragma unroll
     for (int mt = 0; mt < PW_MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < PW_NT; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
 
@@ -147,12 +149,13 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
     }
     __syncthreads();
 
-    // B fragments: lane = pixel pair q, k rows 8 ko .. 8 ko + 7 of a 16-row sub-step.  The raw words of the next
+    // B fragments: lane = pixel group q (NT pixels), k rows 8 ko .. 8 ko + 7 of a 16-row sub-step.  The raw words of the next
     // sub-step are read while the MFMAs of the current one run (hence three stages: chunk c + 1 is read during chunk c).
-    const unsigned char* fragbase = &lds[0] + (8 * ko) * PITCH + (pxw + 2 * q) * 2;
-    unsigned int rw[8];
+    typedef unsigned int rw_t __attribute__((ext_vector_type(NT / 2)));
+    const unsigned char* fragbase = &lds[0] + (8 * ko) * PITCH + (pxw + NT * q) * 2;
+    rw_t rw[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const unsigned int*>(fragbase + r * PITCH);
+    for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const rw_t*>(fragbase + r * PITCH);
     int s0 = 0;                                    // stage of chunk c
     for (int c0 = 0; c0 < nchunks; c0 += D) {
 #pragma unroll
@@ -162,20 +165,22 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
             const int s2 = (s1 == 2) ? 0 : s1 + 1; // stage of chunk c + 2
 #pragma unroll
             for (int ks = 0; ks < PW_KS; ++ks) {
-                u32x4 bf[PW_NT];
+                u32x4 bf[NT];
 #pragma unroll
-                for (int h = 0; h < 4; ++h) {
-                    bf[0][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x05040100u);
-                    bf[1][h] = __builtin_amdgcn_perm(rw[2 * h + 1], rw[2 * h], 0x07060302u);
-                }
+                for (int pp = 0; pp < NT / 2; ++pp)
+#pragma unroll
+                    for (int h = 0; h < 4; ++h) {
+                        bf[2 * pp][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x05040100u);
+                        bf[2 * pp + 1][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x07060302u);
+                    }
                 const unsigned char* fb = (ks + 1 < PW_KS) ? fragbase + s0 * STAGE + (ks + 1) * PW_KC * PITCH : fragbase + s1 * STAGE;
 #pragma unroll
-                for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const unsigned int*>(fb + r * PITCH);
+                for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const rw_t*>(fb + r * PITCH);
 #pragma unroll
                 for (int mt = 0; mt < PW_MT; ++mt) {
                     const bf16x8 av = __builtin_bit_cast(bf16x8, araw[u][ks][mt]);
 #pragma unroll
-                    for (int t = 0; t < PW_NT; ++t)
+                    for (int t = 0; t < NT; ++t)
                         acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
                 }
             }
@@ -188,20 +193,20 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
         }
     }
 
-    // epilogue: lane holds rows 8 (v / 4) + 4 ko + v % 4 of each 32-row tile and pixels 2 q, 2 q + 1
-    const int64_t px = pw0 + pxw + 2 * q;
+    // epilogue: lane holds rows 8 (v / 4) + 4 ko + v % 4 of each 32-row tile and pixels NT q .. NT q + NT - 1
+    const int64_t px = pw0 + pxw + NT * q;
     if (px >= a.P) return;
     unsigned short* __restrict__ Y = a.Y + (int64_t)b * a.O * a.P;
     const unsigned short* __restrict__ R = a.addend ? a.addend + (int64_t)b * a.O * a.P : nullptr;
 #pragma unroll
     for (int mt = 0; mt < PW_MT; ++mt) {
-        unsigned int rv[16];
+        rw_t rv[16];
         if (R) {
             // all addend loads of the tile first
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int o = min(o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3), a.O - 1);
-                rv[v] = *reinterpret_cast<const unsigned int*>(R + (int64_t)o * a.P + px);
+                rv[v] = *reinterpret_cast<const rw_t*>(R + (int64_t)o * a.P + px);
             }
         }
 #pragma unroll
@@ -209,18 +214,188 @@ __global__ __launch_bounds__(PW_THREADS) void pw_gemm_kernel(PointwiseArgs a) {
             const int o = o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3);
             if (o >= a.O) continue;
             const float bs = a.bias ? a.bias[o] : 0.f;
-            float y0 = acc[mt][0][v] + bs, y1 = acc[mt][1][v] + bs;
+            float y[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) y[t] = acc[mt][t][v] + bs;
             if (a.act == SFNO_ACT_GELU) {
-                y0 = gelu(y0);
-                y1 = gelu(y1);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) y[t] = gelu(y[t]);
             }
             if (R) {
                 const float sc = a.add_scale ? a.add_scale[(int64_t)b * a.O + o] : 1.f;
                 const float sh = a.add_shift ? a.add_shift[(int64_t)b * a.O + o] : 0.f;
-                y0 += fmaf(sc, __uint_as_float(rv[v] << 16), sh);
-                y1 += fmaf(sc, __uint_as_float(rv[v] & 0xffff0000u), sh);
+#pragma unroll
+                for (int pp = 0; pp < NT / 2; ++pp) {
+                    y[2 * pp] += fmaf(sc, __uint_as_float(rv[v][pp] << 16), sh);
+                    y[2 * pp + 1] += fmaf(sc, __uint_as_float(rv[v][pp] & 0xffff0000u), sh);
+                }
             }
-            *reinterpret_cast<unsigned int*>(Y + (int64_t)o * a.P + px) = (unsigned int)f_to_bf16(y0) | ((unsigned int)f_to_bf16(y1) << 16);
+            rw_t out;
+#pragma unroll
+            for (int pp = 0; pp < NT / 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
+            *reinterpret_cast<rw_t*>(Y + (int64_t)o * a.P + px) = out;
+        }
+    }
+}
+
+// ---- tall variant with direct-to-LDS loads ----------------------------------------------------------
+// For O > 96 the kernel above is bound by the weight fragments every wavefront pulls through L1 for only 6 MFMAs
+// each.  This variant gives a wavefront 96 rows x 128 pixels (3 x 4 tiles, 192 accumulator registers), eight
+// wavefronts per workgroup (384 rows x 256 pixels, half the weight traffic per pixel), and moves both operand
+// streams with global_load_lds_dwordx4: lane i's 16 bytes land at LDS base + 16 i, no staging registers, so three
+// stages of 32 k rows (40 KiB each) give a two-chunk prefetch distance within the 256 registers two wavefronts
+// per SIMD leave.  The loads are issued from inline assembly: the compiler would otherwise order every LDS read
+// behind all outstanding direct-to-LDS loads; the waits are written out by hand (5 loads per wavefront and chunk).
+constexpr int DM_MT = 3, DM_NT = 4;
+constexpr int DM_ROWS = 4 * 32 * DM_MT;          // 384 rows per workgroup
+constexpr int DM_PX = 2 * 32 * DM_NT;            // 256 pixels per workgroup
+constexpr int DM_CK = 32;                        // k rows per chunk
+constexpr int DM_ABYTES = 2 * (DM_ROWS / 32) * 1024;   // 24 fragment blocks of 1 KiB
+constexpr int DM_XBLK = 1024 + 16;               // two pixel rows of the chunk (2 x 512 bytes) + padding
+constexpr int DM_STAGE = DM_ABYTES + (DM_CK / 2) * DM_XBLK;
+constexpr int DM_NSTAGE = 3;
+
+__device__ __forceinline__ void dma16(const void* g, unsigned lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_addr) : "memory");
+}
+
+__global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
+    __shared__ __align__(16) unsigned char lds[DM_NSTAGE * DM_STAGE];
+    const int xcd = blockIdx.x & 7, qid = blockIdx.x >> 3;
+    const int ob = qid % a.n_oblk;
+    const int64_t strip_lin = (int64_t)(qid / a.n_oblk) * 8 + xcd;
+    if (strip_lin >= a.n_strips * a.B) return;
+    const int b = (int)(strip_lin / a.n_strips);
+    const int64_t pw0 = (strip_lin - (int64_t)b * a.n_strips) * DM_PX;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wo = wave >> 1, wp = wave & 1;                    // 4 wavefronts along the rows x 2 along the pixels
+    const int q = lane & 31, ko = lane >> 5;
+    const int o0 = ob * DM_ROWS + wo * 32 * DM_MT;
+    const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)lds);
+
+    // this wavefront's share of a chunk: weight blocks (k step wave >> 2, row blocks 3 (wave & 3) .. + 2) and
+    // activation blocks 2 wave, 2 wave + 1 (block = rows 2 xb, 2 xb + 1 of the chunk; lane = row (lane >> 5), 8 pixels (lane & 31))
+    const int nc16 = a.Kpad / PW_KC;
+    const int nchunks = a.Kpad / DM_CK;
+    const unsigned short* wsrc = a.W + (((int64_t)(ob * (DM_ROWS / 32) + 3 * (wave & 3)) * nc16 + (wave >> 2)) * 64 + lane) * 8;
+    const int64_t wrb = (int64_t)nc16 * 512;                   // ushorts between row blocks
+    const unsigned short* __restrict__ X = a.X + (int64_t)b * a.K * a.P + min(pw0 + 8 * (lane & 31), a.P - 8);
+    const int xrow0 = 4 * wave + (lane >> 5);                   // first of this lane's rows in the chunk: 2 (2 wave + i) + (lane >> 5)
+
+    auto issue = [&](int c, int stage) {
+        const unsigned sb = lds0 + stage * DM_STAGE;
+        const unsigned short* wp_ = wsrc + (int64_t)c * 1024;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) dma16(wp_ + i * wrb, sb + ((wave >> 2) * 12 + 3 * (wave & 3) + i) * 1024);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int k = min(c * DM_CK + xrow0 + 2 * i, a.K - 1);      // rows past K meet zero weights
+            dma16(X + (int64_t)k * a.P, sb + DM_ABYTES + (2 * wave + i) * DM_XBLK);
+        }
+    };
+
+    f32x16 acc[DM_MT][DM_NT];
+#pragma unroll
+    for (int mt = 0; mt < DM_MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < DM_NT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
+
+    issue(0, 0);
+    if (nchunks > 1) {
+        issue(1, 1);
+        __builtin_amdgcn_s_waitcnt(0x0F75);        // vmcnt(5): chunk 0 has landed
+    } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
+    }
+    __syncthreads();
+
+    const unsigned char* abase = lds + (DM_MT * wo) * 1024 + lane * 16;
+    const unsigned char* xbase = lds + DM_ABYTES + (4 * ko) * DM_XBLK + wp * 256 + 8 * q;
+    int stage = 0;
+    for (int c = 0; c < nchunks; ++c) {
+        const int s2 = (stage == 0) ? 2 : stage - 1;            // (stage + 2) % 3
+        if (c + 2 < nchunks) issue(c + 2, s2);
+        const unsigned char* sa = abase + stage * DM_STAGE;
+        const unsigned char* sx = xbase + stage * DM_STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            u32x2 rw[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const u32x2*>(sx + (8 * ks + (r >> 1)) * DM_XBLK + (r & 1) * 512);
+            u32x4 af[DM_MT];
+#pragma unroll
+            for (int mt = 0; mt < DM_MT; ++mt) af[mt] = *reinterpret_cast<const u32x4*>(sa + (ks * 12 + mt) * 1024);
+            u32x4 bf[DM_NT];
+#pragma unroll
+            for (int pp = 0; pp < 2; ++pp)
+#pragma unroll
+                for (int h = 0; h < 4; ++h) {
+                    bf[2 * pp][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x05040100u);
+                    bf[2 * pp + 1][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x07060302u);
+                }
+#pragma unroll
+            for (int mt = 0; mt < DM_MT; ++mt) {
+                const bf16x8 av = __builtin_bit_cast(bf16x8, af[mt]);
+#pragma unroll
+                for (int t = 0; t < DM_NT; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+            }
+        }
+        // chunk c + 1 (issued one iteration ago) must have landed for every wavefront before it is read, and every
+        // wavefront must be done with this stage before chunk c + 3 overwrites it
+        if (c + 2 < nchunks)
+            __builtin_amdgcn_s_waitcnt(0x0F75);    // vmcnt(5): all but the loads of chunk c + 2
+        else
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        stage = (stage == 2) ? 0 : stage + 1;
+    }
+
+    // epilogue: lane holds rows 8 (v / 4) + 4 ko + v % 4 of each 32-row tile and pixels 4 q .. 4 q + 3
+    const int64_t px = pw0 + wp * 128 + 4 * q;
+    if (px >= a.P) return;
+    unsigned short* __restrict__ Y = a.Y + (int64_t)b * a.O * a.P;
+    const unsigned short* __restrict__ R = a.addend ? a.addend + (int64_t)b * a.O * a.P : nullptr;
+#pragma unroll
+    for (int mt = 0; mt < DM_MT; ++mt) {
+        if (o0 + 32 * mt >= a.O) break;
+        u32x2 rv[16];
+        if (R) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int o = min(o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3), a.O - 1);
+                rv[v] = *reinterpret_cast<const u32x2*>(R + (int64_t)o * a.P + px);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int o = o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3);
+            if (o >= a.O) continue;
+            const float bs = a.bias ? a.bias[o] : 0.f;
+            float y[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) y[t] = acc[mt][t][v] + bs;
+            if (a.act == SFNO_ACT_GELU) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) y[t] = gelu(y[t]);
+            }
+            if (R) {
+                const float sc = a.add_scale ? a.add_scale[(int64_t)b * a.O + o] : 1.f;
+                const float sh = a.add_shift ? a.add_shift[(int64_t)b * a.O + o] : 0.f;
+#pragma unroll
+                for (int pp = 0; pp < 2; ++pp) {
+                    y[2 * pp] += fmaf(sc, __uint_as_float(rv[v][pp] << 16), sh);
+                    y[2 * pp + 1] += fmaf(sc, __uint_as_float(rv[v][pp] & 0xffff0000u), sh);
+                }
+            }
+            u32x2 out;
+#pragma unroll
+            for (int pp = 0; pp < 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
+            *reinterpret_cast<u32x2*>(Y + (int64_t)o * a.P + px) = out;
         }
     }
 }
@@ -351,16 +526,17 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
     if (a.P % 8 != 0 || a.K < 1 || a.O < 1 || a.B < 1 || a.P < 8) return SFNO_EUNSUPPORTED;
     const bool tall = a.O > PW_ROWS;              // several wavefronts share a pixel strip
     const int wm = tall ? 4 : 1;
-    const int wpx = (8 / wm) * PW_PX;
+    const bool dma = tall;                        // direct-to-LDS kernel for O > 96
+    const int wpx = dma ? DM_PX : 512;            // pixels per workgroup
     a.n_oblk = (a.O + PW_ROWS * wm - 1) / (PW_ROWS * wm);
     a.n_strips = (a.P + wpx - 1) / wpx;
     const int64_t strips = a.n_strips * a.B;
     const int64_t blocks = (strips + 7) / 8 * 8 * a.n_oblk;
     if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    if (tall)
-        hipLaunchKernelGGL((pw_gemm_kernel<4>), dim3((unsigned)blocks), dim3(PW_THREADS), 0, s, a);
+    if (dma)
+        hipLaunchKernelGGL(pw_gemm_dma_kernel, dim3((unsigned)blocks), dim3(512), 0, s, a);
     else
-        hipLaunchKernelGGL((pw_gemm_kernel<1>), dim3((unsigned)blocks), dim3(PW_THREADS), 0, s, a);
+        hipLaunchKernelGGL((pw_gemm_kernel<1, 2>), dim3((unsigned)blocks), dim3(512), 0, s, a);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

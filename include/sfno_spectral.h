@@ -207,6 +207,18 @@ size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int 
 int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y, int batch, int mmax,
                 int triangular, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- "diagonal" operator ------------------------------------------------------------- */
+
+/* y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l,m] (makani/models/common/contractions.py:121-127, operator_type
+ * "diagonal"): x complex64 [B][I][P], weight complex64 [I][O][P], y complex64 [B][O][P], P = lmax*mmax
+ * contiguous.  `adjoint` != 0 computes the input gradient instead: x is then the output gradient
+ * [B][O][P] and y[b,i,p] = sum_o x[b,o,p] conj(w[i,o,p]). */
+int sfno_diagonal_contract(const void* x, const void* weight, void* y, int batch, int in_channels,
+                           int out_channels, int64_t positions, int adjoint, void* stream);
+/* gweight[i,o,p] = sum_b conj(x[b,i,p]) gy[b,o,p] */
+int sfno_diagonal_weight_grad(const void* x, const void* gy, void* gweight, int batch, int in_channels,
+                              int out_channels, int64_t positions, void* stream);
+
 /* ---- pointwise tail of the SFNO block (bf16 activations) -------------------------------- */
 
 /* 1x1 convolution on NCHW bfloat16 activations with a fused epilogue:

@@ -434,6 +434,22 @@ extern "C" int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y,
     return sfno_spectral_to_coeffs(sout, y, (int64_t)batch * w->O, w->L, mmax, triangular, stream);
 }
 
+// ---- diagonal operator -----------------------------------------------------------------------------
+
+extern "C" int sfno_diagonal_contract(const void* x, const void* weight, void* y, int batch, int in_channels, int out_channels,
+                                      int64_t positions, int adjoint, void* stream) {
+    if (!x || !weight || !y || batch < 1 || in_channels < 1 || out_channels < 1 || positions < 1) return SFNO_EINVAL;
+    return diagonal_contract_launch(reinterpret_cast<const float2*>(x), reinterpret_cast<const float2*>(weight), reinterpret_cast<float2*>(y),
+                                    batch, in_channels, out_channels, positions, adjoint ? 1 : 0, (hipStream_t)stream);
+}
+
+extern "C" int sfno_diagonal_weight_grad(const void* x, const void* gy, void* gweight, int batch, int in_channels, int out_channels,
+                                         int64_t positions, void* stream) {
+    if (!x || !gy || !gweight || batch < 1 || in_channels < 1 || out_channels < 1 || positions < 1) return SFNO_EINVAL;
+    return diagonal_wgrad_launch(reinterpret_cast<const float2*>(x), reinterpret_cast<const float2*>(gy), reinterpret_cast<float2*>(gweight), batch,
+                                 in_channels, out_channels, positions, (hipStream_t)stream);
+}
+
 // ---- pointwise tail -----------------------------------------------------------------------------
 
 extern "C" int64_t sfno_pointwise_weight_elems(int O, int K) {

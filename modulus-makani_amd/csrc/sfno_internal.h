@@ -63,6 +63,10 @@ struct DhconvWgradArgs {
 };
 int dhconv_wgrad_launch(const DhconvWgradArgs& a, hipStream_t s);
 
+// ---- "diagonal" operator on the reference layout (diagonal.hip): x [B][I][P], w [I][O][P], y [B][O][P], P = L*M ----
+int diagonal_contract_launch(const float2* x, const float2* w, float2* y, int B, int I, int O, int64_t P, int adjoint, hipStream_t s);
+int diagonal_wgrad_launch(const float2* x, const float2* g, float2* gw, int B, int I, int O, int64_t P, hipStream_t s);
+
 // ---- pointwise tail (pointwise.hip): bf16 NCHW activations, 1x1 convolutions on bf16 MFMA ------------
 struct PointwiseArgs {
     const unsigned short* X;       // bf16 [B][K][P]

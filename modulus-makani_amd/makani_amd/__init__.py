@@ -1,10 +1,10 @@
 """MI355X-native SFNO spectral hot path: RealSHT / InverseRealSHT / SpectralConv (dhconv)
 on hand-written HIP kernels behind the C ABI of include/sfno_spectral.h."""
 from .sht import RealSHT, InverseRealSHT, quadrature, legendre_table, legendre_gauss_weights, clenshaw_curtiss_weights, lobatto_weights
-from .contractions import _contract_dhconv, get_contract_fun, dhconv_spectral
+from .contractions import _contract_dhconv, _contract_diagonal, get_contract_fun, dhconv_spectral
 from .spectral_convolution import SpectralConv
 
 __all__ = [
     "RealSHT", "InverseRealSHT", "SpectralConv", "quadrature", "legendre_table", "legendre_gauss_weights",
-    "clenshaw_curtiss_weights", "lobatto_weights", "_contract_dhconv", "get_contract_fun", "dhconv_spectral",
+    "clenshaw_curtiss_weights", "lobatto_weights", "_contract_dhconv", "_contract_diagonal", "get_contract_fun", "dhconv_spectral",
 ]

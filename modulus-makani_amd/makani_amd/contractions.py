@@ -191,14 +191,62 @@ def _dhconv(ac, bc, triangular, compute, adjoint):
     return out
 
 
+class _DiagonalFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ac, bc):
+        ctx.save_for_backward(ac, bc)
+        return _diagonal(ac, bc, False)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, g):
+        ac, bc = ctx.saved_tensors
+        g = g.contiguous()
+        B, I, L, M = ac.shape
+        O = bc.shape[1]
+        gac = gbc = None
+        if ctx.needs_input_grad[0]:
+            gac = _diagonal(g, bc, True)
+        if ctx.needs_input_grad[1]:
+            gbc = torch.zeros_like(bc)
+            if g.numel():
+                check(lib.sfno_diagonal_weight_grad(ctypes.c_void_p(ac.data_ptr()), ctypes.c_void_p(g.data_ptr()), ctypes.c_void_p(gbc.data_ptr()),
+                                                    B, I, O, L * M, _stream(ac.device)), "sfno_diagonal_weight_grad")
+        return gac, gbc
+
+
+def _diagonal(ac, bc, adjoint):
+    B, _, L, M = ac.shape
+    I, O = bc.shape[0], bc.shape[1]
+    out = torch.empty((B, I if adjoint else O, L, M), dtype=torch.complex64, device=ac.device)
+    if out.numel():
+        check(lib.sfno_diagonal_contract(ctypes.c_void_p(ac.data_ptr()), ctypes.c_void_p(bc.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                                         B, I, O, L * M, int(adjoint), _stream(ac.device)), "sfno_diagonal_contract")
+    return out
+
+
+def _contract_diagonal(ac: torch.Tensor, bc: torch.Tensor) -> torch.Tensor:
+    """einsum("bixy,ioxy->boxy") on complex64 tensors (contractions.py:121-127)."""
+    if ac.dim() != 4 or bc.dim() != 4 or ac.shape[1] != bc.shape[0] or ac.shape[2:] != bc.shape[2:]:
+        raise RuntimeError(f"diagonal: shapes {tuple(ac.shape)} and {tuple(bc.shape)} do not match 'bixy,ioxy->boxy'")
+    if ac.dtype != torch.complex64 or bc.dtype != torch.complex64:
+        raise TypeError(f"diagonal contraction computes in complex64, got {ac.dtype} and {bc.dtype}")
+    if ac.device.type != "cuda":
+        raise RuntimeError("the diagonal contraction kernel runs on a HIP device only")
+    return _DiagonalFn.apply(ac.contiguous(), bc.contiguous())
+
+
 def _contract_dense(x, weight, separable=False, operator_type="diagonal", complex=True):
-    """Mirror of _contract_dense_pytorch (factorizations.py:167-200) for the operator this library implements."""
-    if operator_type == "diagonal":
-        raise NotImplementedError("only operator_type='dhconv' runs on the HIP path")
-    if operator_type != "dhconv":
+    """Mirror of _contract_dense_pytorch (factorizations.py:167-200).
+
+    The separable variants are not provided: the reference's einsums for them ("bixy,ixy->boxy", "bixy,ix->boxy",
+    contractions.py:139-154) name an output index that no input carries, so they cannot be evaluated there either."""
+    if operator_type not in ("diagonal", "dhconv"):
         raise ValueError(f"Unkonw operator type {operator_type}")
     if separable or not complex:
-        raise NotImplementedError("only the non-separable complex dhconv runs on the HIP path")
+        raise NotImplementedError("only the non-separable complex operators run on the HIP path")
+    if operator_type == "diagonal":
+        return _contract_diagonal(x, weight)
     return _contract_dhconv(x, weight)
 
 

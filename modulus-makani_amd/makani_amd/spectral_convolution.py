@@ -46,8 +46,8 @@ class SpectralConv(nn.Module):
             weight_shape += [self.modes_lat_local]
         else:
             raise ValueError(f"Unsupported operator type f{self.operator_type}")
-        if self.operator_type != "dhconv" or self.separable:
-            raise NotImplementedError("the HIP path implements the non-separable 'dhconv' operator")
+        if self.separable:
+            raise NotImplementedError("the HIP path implements the non-separable operators")
 
         # same initialisation as the reference (spectral_convolution.py:97-102)
         scale = math.sqrt(gain / in_channels) * torch.ones(self.modes_lat_local, dtype=torch.complex64)
@@ -63,7 +63,8 @@ class SpectralConv(nn.Module):
             self.bias = nn.Parameter(torch.zeros(1, self.out_channels, self.nlat_local, self.nlon_local))
 
         self._fused = (
-            isinstance(forward_transform, RealSHT)
+            operator_type == "dhconv"
+            and isinstance(forward_transform, RealSHT)
             and isinstance(inverse_transform, InverseRealSHT)
             and forward_transform.lmax == inverse_transform.lmax
             and forward_transform.mmax == inverse_transform.mmax

@@ -18,6 +18,14 @@ def dhconv(x, w):
     return np.einsum("bixy,iox->boxy", x, w, optimize=True)
 
 
+def diagonal(x, w):
+    """y[b,o,l,m] = sum_i x[b,i,l,m] * w[i,o,l,m] (makani/models/common/contractions.py:121-127)."""
+    x = np.asarray(x)
+    w = np.asarray(w)
+    assert x.shape[1] == w.shape[0] and x.shape[2:] == w.shape[2:]
+    return np.einsum("bixy,ioxy->boxy", x, w, optimize=True)
+
+
 def spectral_conv(x, w, fwd_tables, inv_tables, bias=None):
     """Returns (y, residual) as SpectralConv.forward does, all in float64.
 
@@ -29,10 +37,11 @@ def spectral_conv(x, w, fwd_tables, inv_tables, bias=None):
         fwd_tables.nlat != inv_tables.nlat or fwd_tables.nlon != inv_tables.nlon or fwd_tables.grid != inv_tables.grid
     )
     residual = np.asarray(x, dtype=np.float64)
+    contract = diagonal if np.asarray(w).ndim == 4 else dhconv
     c = sht_forward(x, fwd_tables)
     if scale_residual:
         residual = sht_inverse(c, inv_tables)
-    y = dhconv(c, np.asarray(w, dtype=np.complex128))
+    y = contract(c, np.asarray(w, dtype=np.complex128))
     y = sht_inverse(y, inv_tables)
     if bias is not None:
         y = y + bias

@@ -104,3 +104,47 @@ def test_contract_dhconv_bf16(lib_built, B, I, O, L, M):
     wb = torch.view_as_complex(torch.view_as_real(w).to(torch.bfloat16).float())
     ref_b = dhconv(xb.numpy().astype(np.complex128), wb.numpy().astype(np.complex128))
     assert rel_l2(got.cpu().numpy(), ref_b) < 1e-5
+
+
+@pytest.mark.parametrize("B,I,O,L,M", [(1, 3, 2, 4, 5), (2, 8, 8, 6, 7), (5, 17, 5, 12, 9), (1, 32, 48, 33, 34), (6, 4, 3, 7, 7)])
+def test_contract_diagonal_and_its_gradients(lib_built, B, I, O, L, M):
+    """operator_type "diagonal" (contractions.py:121-127): values against the oracle, gradients against float64 autograd
+    of the same einsum (odd L*M exercises the unaligned path, B > 4 the batch loop)."""
+    import makani_amd as ma
+    from oracle.dhconv import diagonal
+
+    print(f"case diagonal B={B} I={I} O={O} L={L} M={M}", flush=True)
+    torch.manual_seed(3)
+    x = torch.randn(B, I, L, M, dtype=torch.complex64)
+    w = torch.randn(I, O, L, M, dtype=torch.complex64) / np.sqrt(I)
+    g = torch.randn(B, O, L, M, dtype=torch.complex64)
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    y = ma._contract_diagonal(xg, wg)
+    y.backward(g.cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(y.detach().cpu().numpy(), diagonal(x.numpy().astype(np.complex128), w.numpy().astype(np.complex128))) < TOL
+    xr, wr = x.to(torch.complex128).requires_grad_(True), w.to(torch.complex128).requires_grad_(True)
+    torch.einsum("bixy,ioxy->boxy", xr, wr).backward(g.to(torch.complex128))
+    assert rel_l2(xg.grad.cpu().numpy(), xr.grad.numpy()) < TOL
+    assert rel_l2(wg.grad.cpu().numpy(), wr.grad.numpy()) < TOL
+    f = ma.get_contract_fun(wg, implementation="factorized", separable=False, complex=True, operator_type="diagonal")
+    assert torch.equal(f(xg.detach(), wg.detach(), separable=False, operator_type="diagonal"), y.detach())
+
+
+def test_spectral_conv_diagonal(lib_built):
+    """SpectralConv with operator_type="diagonal" against the oracle (weight [I, O, L, M], lmax == mmax as the
+    reference's initialisation requires)."""
+    import makani_amd as ma
+
+    torch.manual_seed(4)
+    fwd = ma.RealSHT(16, 32, lmax=12, mmax=12, grid="legendre-gauss")
+    inv = ma.InverseRealSHT(16, 32, lmax=12, mmax=12, grid="legendre-gauss")
+    conv = ma.SpectralConv(fwd, inv, 5, 3, operator_type="diagonal").cuda()
+    assert tuple(conv.weight.shape) == (5, 3, 12, 12)
+    x = torch.randn(2, 5, 16, 32)
+    y, res = conv(x.cuda())
+    torch.cuda.synchronize()
+    t = ShtTables(16, 32, 12, 12, "legendre-gauss")
+    ref, _ = spectral_conv(x.double().numpy(), conv.weight.detach().cpu().numpy().astype(np.complex128), t, t)
+    assert rel_l2(y.detach().cpu().numpy(), ref) < TOL
+    assert torch.equal(res, x.cuda())

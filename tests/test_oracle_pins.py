@@ -253,6 +253,26 @@ def test_dhconv_brute_force():
     assert np.allclose(dhconv(x[:, :, :1], w[:, :, :1])[:, :, 0], np.einsum("bim,io->bom", x[:, :, 0], w[:, :, 0]))
 
 
+def test_diagonal_brute_force():
+    from oracle.dhconv import diagonal
+
+    rng = np.random.default_rng(10)
+    B, I, O, L, M = 2, 3, 4, 5, 6
+    x = rng.standard_normal((B, I, L, M)) + 1j * rng.standard_normal((B, I, L, M))
+    w = rng.standard_normal((I, O, L, M)) + 1j * rng.standard_normal((I, O, L, M))
+    y = np.zeros((B, O, L, M), dtype=complex)
+    for b in range(B):
+        for o in range(O):
+            for l in range(L):
+                for m in range(M):
+                    for i in range(I):
+                        y[b, o, l, m] += x[b, i, l, m] * w[i, o, l, m]
+    assert np.allclose(diagonal(x, w), y, atol=1e-13)
+    # a weight that does not depend on m is the dhconv operator
+    wl = w[:, :, :, :1]
+    assert np.allclose(diagonal(x, np.broadcast_to(wl, w.shape)), dhconv(x, wl[..., 0]), atol=1e-13)
+
+
 def test_spectral_conv_residual_rule():
     rng = np.random.default_rng(9)
     same = ShtTables(12, 24, 12, 13, "legendre-gauss")

@@ -1,18 +1,19 @@
 // dhconv on fp32 MFMA (v_mfma_f32_32x32x2_f32), gfx950.
 //
 //   y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l]        (makani/models/common/contractions.py:130-136)
-// runs as one real GEMM per degree l on the spectral layout,
-//   out[(m,b)][o'] = sum_i' in[(m,b)][i'] * Wt[l][i'][o'],   i' = 2i + {re,im}, o' = 2o + {re,im},
-// where Wt is the 2x2 real embedding of each complex weight: rows 2i, 2i+1 of column pair
-// (2o, 2o+1) are (re, im) and (-im, re).
+// runs as real GEMMs per degree l on the spectral layout.  A complex product costs three real ones
+// (Gauss):  k1 = wr (xr + xi),  k2 = xr (wi - wr),  k3 = xi (wr + wi),  yr = k1 - k3,  yi = k1 + k2,
+// so each complex input channel feeds three MFMA operand pairs instead of the four of the 2x2 real
+// embedding, and a wavefront keeps three accumulators (K1, K2, K3) per tile that are combined when the
+// rows are stored.
 //
-// A workgroup owns (degree l, block of 128 output columns o', group of 128 rows (m,b)).
-// Each of its four wavefronts owns 32 rows: it reads its own activation rows straight from
-// HBM/L2 into MFMA A-fragments (rows are contiguous along i' in the spectral layout) and
-// keeps a 32 x 128 accumulator.  The weight chunk (16 i' x 128 o') is expanded from the
-// packed complex weights into LDS once per chunk and shared by the four wavefronts as the
-// B operand.  Wavefronts whose rows lie beyond the orders present at this degree (m > l)
-// exit early, so the triangular structure costs no guarded matrix instructions.
+// A workgroup owns (degree l, block of 64 output channels, group of 128 rows (m,b)).  Each of its four
+// wavefronts owns 32 rows: it reads its own activation rows straight from HBM/L2 into MFMA A operands
+// (rows are contiguous along i in the spectral layout) and keeps 32 rows x 64 channels x 3 sums.  The
+// weight chunk (8 input channels x 64 output channels) is expanded from the packed complex weights into
+// three LDS planes (wr, wi - wr, wr + wi) once per chunk and shared by the four wavefronts as the B
+// operand.  Wavefronts whose rows lie beyond the orders present at this degree (m > l) do nothing, so the
+// triangular structure costs no guarded matrix instructions.
 #include <type_traits>
 
 #include "sfno_internal.h"
@@ -25,10 +26,10 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 
 // grid = (8 * ceil(L/8) * nob, row groups); VEC4: 2*I is a multiple of 4 so activation rows can be read as float4
 template <bool VEC4>
-__global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
-    constexpr int NT = DH_COLS / 32;                 // 4 column tiles per wavefront
-    constexpr int LDW = DH_COLS + 32;                // pitch = 32 mod 64: the two half-waves read different banks
-    __shared__ __align__(16) float ws[2][PG_KC][LDW];
+__global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
+    constexpr int NT = DH_COLS / 64;                 // 2 tiles of 32 output channels per wavefront
+    constexpr int LDW = DH_COLS / 2 + 32;            // plane pitch = 32 mod 64: the two half-waves read different banks
+    __shared__ __align__(16) float ws[2][3][8][LDW]; // [buffer][plane][input channel of the chunk][output channel]
 
     // Workgroups go to the 8 XCDs round-robin by linear id: all column blocks and row groups of a
     // degree share their activation panel, so a degree stays on one XCD.  Degrees are handed out
@@ -44,14 +45,14 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
     const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;      // rows (m,b) present at this degree
     const int r0 = blockIdx.y * 128;
     if (r0 >= ncols) return;
-    // Row blocks of 32 present in this group; when there are only one or two (low degrees), the four
-    // wavefronts split the column tiles of those blocks instead of idling.
+    // Row blocks of 32 present in this group; when there are only one or two (low degrees), pairs of
+    // wavefronts split the two column tiles of a block instead of idling.
     const int nrb = min(4, (ncols - r0 + 31) / 32);
-    const int ntw = nrb == 1 ? 1 : (nrb == 2 ? 2 : 4);                 // column tiles per wavefront
-    const int rb = nrb == 1 ? 0 : (nrb == 2 ? (wave >> 1) : wave);     // my row block
-    const int t0 = nrb == 1 ? wave : (nrb == 2 ? 2 * (wave & 1) : 0);  // my first column tile
+    const bool split = nrb <= 2;
+    const int rb = split ? (wave >> 1) : wave;       // my row block
+    const int t0 = split ? (wave & 1) : 0;           // my first column tile
     const bool active = rb < nrb;
-    const int nc = a.nc;                                           // K chunks of 16 i' (8 complex input channels)
+    const int nc = a.nc;                             // K chunks of 8 complex input channels
     const int kh = lane >> 5, cl = lane & 31;
 
     // my activation row (clamped: rows past the end repeat the last one and are not stored)
@@ -61,17 +62,20 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
     // packed weights of (l, ob): nc chunks of 8 x 64 complex, 16 bytes per thread and chunk
     const f4* wp = reinterpret_cast<const f4*>(a.W) + ((int64_t)l * a.nob + ob) * nc * 256 + tid;
 
-    floatx16 acc[NT];
+    floatx16 acc[3][NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int p = 0; p < 3; ++p)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[p][t][v] = 0.0f;
 
-    // A fragments: lane (row, kh) holds i' = 16c + 8kh .. +7; k-step s of the chunk uses i' = 16c + 8kh + s
-    // on both operands.  Reads are clamped into the row; the weights are zero beyond 2*I.
+    // A operands: lane (row, kh) holds the complex channels i = 8c + 4kh + s, s = 0..3, as (re, im) pairs; k-step s
+    // of the chunk uses channel 4kh + s of the chunk on both operands.  Reads are clamped into the row; the weights
+    // are zero beyond I.
     auto x_load = [&](int c, f4 (&xr)[2]) {
         if (VEC4) {
-            // a group of four i' is either entirely inside the row or entirely in the zero-weight padding
+            // a group of two channels is either entirely inside the row or entirely in the zero-weight padding
             const int k = 16 * c + 8 * kh;
             xr[0] = *reinterpret_cast<const f4*>(xrow + min(k, a.I2 - 4));
             xr[1] = *reinterpret_cast<const f4*>(xrow + min(k + 4, a.I2 - 4));
@@ -85,28 +89,32 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
             }
         }
     };
-    // thread t expands complex pair (i = t/32, o = 2(t%32), 2(t%32)+1) of the chunk
+    // thread t expands the complex pair (i = t/32, o = 2(t%32), 2(t%32)+1) of the chunk into the three planes
     auto w_store = [&](int buf, f4 w) {
         const int ii = tid >> 5, o2 = tid & 31;
-        *reinterpret_cast<f4*>(&ws[buf][2 * ii][4 * o2]) = w;
-        const f4 r = {-w[1], w[0], -w[3], w[2]};
-        *reinterpret_cast<f4*>(&ws[buf][2 * ii + 1][4 * o2]) = r;
+        *reinterpret_cast<f2*>(&ws[buf][0][ii][2 * o2]) = f2{w[0], w[2]};
+        *reinterpret_cast<f2*>(&ws[buf][1][ii][2 * o2]) = f2{w[1] - w[0], w[3] - w[2]};
+        *reinterpret_cast<f2*>(&ws[buf][2][ii][2 * o2]) = f2{w[0] + w[1], w[2] + w[3]};
     };
     // one K-chunk of MFMAs over TI column tiles starting at tile t0; no branches inside
     auto compute_n = [&](auto ti, int buf, const f4 (&xr)[2]) {
         constexpr int TI = decltype(ti)::value;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const float* wrow = &ws[buf][8 * kh + s][32 * t0 + cl];
-            const float xv = xr[s >> 2][s & 3];
+        for (int s = 0; s < 4; ++s) {
+            const float re = xr[s >> 1][2 * (s & 1)], im = xr[s >> 1][2 * (s & 1) + 1];
+            const float sum = re + im;
+            const float* w0 = &ws[buf][0][4 * kh + s][32 * t0 + cl];
 #pragma unroll
-            for (int t = 0; t < TI; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv, wrow[32 * t], acc[t], 0, 0, 0);
+            for (int t = 0; t < TI; ++t) {
+                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(sum, w0[32 * t], acc[0][t], 0, 0, 0);
+                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(re, w0[8 * LDW + 32 * t], acc[1][t], 0, 0, 0);
+                acc[2][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(im, w0[16 * LDW + 32 * t], acc[2][t], 0, 0, 0);
+            }
         }
     };
     auto compute = [&](int buf, const f4 (&xr)[2]) {
-        if (ntw == 4) compute_n(std::integral_constant<int, 4>(), buf, xr);
-        else if (ntw == 2) compute_n(std::integral_constant<int, 2>(), buf, xr);
-        else compute_n(std::integral_constant<int, 1>(), buf, xr);
+        if (split) compute_n(std::integral_constant<int, 1>(), buf, xr);
+        else compute_n(std::integral_constant<int, NT>(), buf, xr);
     };
 
     // software pipeline, one chunk deep; the explicit wait at the end of each iteration keeps
@@ -135,7 +143,8 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
 
     if (!active) return;
     // D layout of the 32x32 MFMA: register v of lane j holds D[8*(v/4) + 4*(j/32) + v%4][j%32];
-    // D rows = my 32 activation rows, D cols = output columns o'
+    // D rows = my 32 activation rows, D cols = output channels; (re, im) = (K1 - K3, K1 + K2)
+    const int ntw = split ? 1 : NT;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int nn = r0 + 32 * rb + 8 * (v >> 2) + 4 * kh + (v & 3);
@@ -144,8 +153,8 @@ __global__ __launch_bounds__(256, 3) void dhconv_kernel(DhconvArgs a) {
         float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int oc = DH_COLS * ob + 32 * (t0 + t) + cl;
-            if (t < ntw && oc < a.O2) orow[oc] = acc[t][v];
+            const int oc = DH_COLS * ob + 2 * (32 * (t0 + t) + cl);
+            if (t < ntw && oc < a.O2) *reinterpret_cast<f2*>(orow + oc) = f2{acc[0][t][v] - acc[2][t][v], acc[0][t][v] + acc[1][t][v]};
         }
     }
 }

@@ -23,7 +23,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 // contraction runs on v_mfma_f32_32x32x16_bf16 with the panel values rounded to bf16 (nearest even) as they are
 // read from LDS; accumulation stays fp32.
 template <int NT, bool ANALYSIS, bool BF16>
-__global__ __launch_bounds__(256, 3) void legendre_fold_kernel(PgemmArgs a) {
+__global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(PgemmArgs a) {
     constexpr int TN = 32 * NT;
     constexpr int LDQ = TN + ((TN % 64 == 0) ? 32 : 0);
     // [buffer][parity][k][column]; reused for the parity exchange of the synthesis epilogue

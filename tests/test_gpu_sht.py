@@ -168,3 +168,20 @@ def test_bf16_compute_variant(lib_built, nlat, nlon, lmax, mmax, grid, lead):
     print(f"   rel-L2 forward {e_fwd:.2e} inverse {e_inv:.2e}", flush=True)
     assert e_fwd < 1e-2 and e_inv < 1e-2
     assert e_fwd > 1e-5 or e_inv > 1e-5          # it is the reduced-precision path that ran
+
+
+def test_known_answers_config0(lib_built):
+    """configs[0] (equiangular 32 x 64, lmax 32, mmax 33, batch 2, 4 channels) against the committed known answers
+    of tests/golden (scipy spherical harmonics, no oracle involved): rel-L2 <= 1e-5 both ways."""
+    import os
+    import makani_amd as ma
+
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "sht_32x64_known_answers.npz"))
+    nlat, nlon, lmax, mmax = int(g["nlat"]), int(g["nlon"]), int(g["lmax"]), int(g["mmax"])
+    fwd = ma.RealSHT(nlat, nlon, lmax, mmax, grid="equiangular")
+    inv = ma.InverseRealSHT(nlat, nlon, lmax, mmax, grid="equiangular")
+    c = fwd(torch.from_numpy(g["x"]).cuda())
+    x = inv(torch.from_numpy(g["coeffs"]).cuda())
+    torch.cuda.synchronize()
+    assert np.linalg.norm(c.cpu().numpy() - g["forward"]) / np.linalg.norm(g["forward"]) < 1e-5
+    assert np.linalg.norm(x.cpu().numpy() - g["inverse"]) / np.linalg.norm(g["inverse"]) < 1e-5

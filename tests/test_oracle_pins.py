@@ -331,3 +331,18 @@ def test_torch_restatement_matches_numpy_oracle_and_its_gradient_is_the_transpos
     ref.inverse(ct).backward(torch.from_numpy(gx))
     want = np.einsum("jlmp,j->lmp", K, gx.ravel())
     np.testing.assert_allclose(torch.view_as_real(ct.grad).numpy(), want, rtol=1e-10, atol=1e-12)
+
+
+def test_oracle_against_committed_known_answers():
+    """tests/golden/sht_32x64_known_answers.npz (made by tests/golden/make_golden.py from scipy's spherical harmonics and
+    moment-equation quadrature weights, without the oracle): smallest benchmark configuration, both directions."""
+    import os
+    from oracle.sht import ShtTables, sht_forward, sht_inverse
+
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "sht_32x64_known_answers.npz"))
+    t = ShtTables(int(g["nlat"]), int(g["nlon"]), int(g["lmax"]), int(g["mmax"]), "equiangular")
+    np.testing.assert_allclose(t.quad_w, g["weights"], rtol=1e-11, atol=1e-14)
+    fwd = sht_forward(g["x"].astype(np.float64), t)
+    assert np.linalg.norm(fwd - g["forward"]) / np.linalg.norm(g["forward"]) < 1e-12
+    inv = sht_inverse(g["coeffs"].astype(np.complex128), t)
+    assert np.linalg.norm(inv - g["inverse"]) / np.linalg.norm(g["inverse"]) < 1e-12

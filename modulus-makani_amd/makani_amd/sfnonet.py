@@ -313,13 +313,14 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
     def _forward_fused(self, x):
         """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""
         enc, dec = _fused_chain(self.encoder.fwd), _fused_chain(self.decoder.fwd)
+        xb = x.to(torch.bfloat16).contiguous()
         if self.big_skip:
             if self.out_shape != self.inp_shape:
-                residual = self.itrans_up(self.trans_down(x.to(torch.float32)).contiguous())
+                residual = self.itrans_up(self.trans_down(x.to(torch.float32)).contiguous()).to(torch.bfloat16).contiguous()
             else:
-                residual = x
-            residual = pw.conv1x1(residual.to(torch.bfloat16).contiguous(), self.residual_transform.weight)
-        x = _run_chain(enc, x.to(torch.bfloat16).contiguous())
+                residual = xb
+            residual = pw.conv1x1(residual, self.residual_transform.weight)
+        x = _run_chain(enc, xb)
         x = self._forward_features(x)
         return _run_chain(dec, x.to(torch.bfloat16).contiguous(), residual if self.big_skip else None)
 

@@ -7,9 +7,10 @@
 // embedding, and a wavefront keeps three accumulators (K1, K2, K3) per tile that are combined when the
 // rows are stored.
 //
-// A workgroup owns (degree l, block of 64 output channels, group of 128 rows (m,b)).  Each of its four
-// wavefronts owns 32 rows: it reads its own activation rows straight from HBM/L2 into MFMA A operands
-// (rows are contiguous along i in the spectral layout) and keeps 32 rows x 64 channels x 3 sums.  The
+// A workgroup owns (degree l, block of 64 output channels, group of 64 rows (m,b)): a small group, because a
+// degree has at most mmax orders and the last group of a degree is rarely full.  Each of its four wavefronts
+// owns 32 rows x 32 output channels: it reads its activation rows straight from HBM/L2 into MFMA A operands
+// (rows are contiguous along i in the spectral layout) and keeps 32 rows x 32 channels x 3 sums.  The
 // weight chunk (8 input channels x 64 output channels) is expanded from the packed complex weights into
 // three LDS planes (wr, wi - wr, wr + wi) once per chunk and shared by the four wavefronts as the B
 // operand.  Wavefronts whose rows lie beyond the orders present at this degree (m > l) do nothing, so the
@@ -25,9 +26,9 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f2 __attribute__((ext_vector_type(2)));
 
 // grid = (8 * ceil(L/8) * nob, row groups); VEC4: 2*I is a multiple of 4 so activation rows can be read as float4
+constexpr int DH_GROUP = 64;                         // rows (m,b) per workgroup
 template <bool VEC4>
-__global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
-    constexpr int NT = DH_COLS / 64;                 // 2 tiles of 32 output channels per wavefront
+__global__ __launch_bounds__(256, 4) void dhconv_kernel(DhconvArgs a) {
     constexpr int LDW = DH_COLS / 2 + 32;            // plane pitch = 32 mod 64: the two half-waves read different banks
     __shared__ __align__(16) float ws[2][3][8][LDW]; // [buffer][plane][input channel of the chunk][output channel]
 
@@ -43,14 +44,11 @@ __global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
     const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;      // rows (m,b) present at this degree
-    const int r0 = blockIdx.y * 128;
+    const int r0 = blockIdx.y * DH_GROUP;
     if (r0 >= ncols) return;
-    // Row blocks of 32 present in this group; when there are only one or two (low degrees), pairs of
-    // wavefronts split the two column tiles of a block instead of idling.
-    const int nrb = min(4, (ncols - r0 + 31) / 32);
-    const bool split = nrb <= 2;
-    const int rb = split ? (wave >> 1) : wave;       // my row block
-    const int t0 = split ? (wave & 1) : 0;           // my first column tile
+    // wavefront = (row block of 32, column tile of 32 output channels)
+    const int nrb = min(DH_GROUP / 32, (ncols - r0 + 31) / 32);
+    const int rb = wave >> 1, t0 = wave & 1;
     const bool active = rb < nrb;
     const int nc = a.nc;                             // K chunks of 8 complex input channels
     const int kh = lane >> 5, cl = lane & 31;
@@ -62,13 +60,11 @@ __global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
     // packed weights of (l, ob): nc chunks of 8 x 64 complex, 16 bytes per thread and chunk
     const f4* wp = reinterpret_cast<const f4*>(a.W) + ((int64_t)l * a.nob + ob) * nc * 256 + tid;
 
-    floatx16 acc[3][NT];
+    floatx16 acc[3];
 #pragma unroll
     for (int p = 0; p < 3; ++p)
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[p][t][v] = 0.0f;
+        for (int v = 0; v < 16; ++v) acc[p][v] = 0.0f;
 
     // A operands: lane (row, kh) holds the complex channels i = 8c + 4kh + s, s = 0..3, as (re, im) pairs; k-step s
     // of the chunk uses channel 4kh + s of the chunk on both operands.  Reads are clamped into the row; the weights
@@ -96,25 +92,17 @@ __global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
         *reinterpret_cast<f2*>(&ws[buf][1][ii][2 * o2]) = f2{w[1] - w[0], w[3] - w[2]};
         *reinterpret_cast<f2*>(&ws[buf][2][ii][2 * o2]) = f2{w[0] + w[1], w[2] + w[3]};
     };
-    // one K-chunk of MFMAs over TI column tiles starting at tile t0; no branches inside
-    auto compute_n = [&](auto ti, int buf, const f4 (&xr)[2]) {
-        constexpr int TI = decltype(ti)::value;
+    // one K-chunk of MFMAs; no branches inside
+    auto compute = [&](int buf, const f4 (&xr)[2]) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const float re = xr[s >> 1][2 * (s & 1)], im = xr[s >> 1][2 * (s & 1) + 1];
             const float sum = re + im;
             const float* w0 = &ws[buf][0][4 * kh + s][32 * t0 + cl];
-#pragma unroll
-            for (int t = 0; t < TI; ++t) {
-                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(sum, w0[32 * t], acc[0][t], 0, 0, 0);
-                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(re, w0[8 * LDW + 32 * t], acc[1][t], 0, 0, 0);
-                acc[2][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(im, w0[16 * LDW + 32 * t], acc[2][t], 0, 0, 0);
-            }
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(sum, w0[0], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(re, w0[8 * LDW], acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(im, w0[16 * LDW], acc[2], 0, 0, 0);
         }
-    };
-    auto compute = [&](int buf, const f4 (&xr)[2]) {
-        if (split) compute_n(std::integral_constant<int, 1>(), buf, xr);
-        else compute_n(std::integral_constant<int, NT>(), buf, xr);
     };
 
     // software pipeline, one chunk deep; the explicit wait at the end of each iteration keeps
@@ -144,18 +132,15 @@ __global__ __launch_bounds__(256, 2) void dhconv_kernel(DhconvArgs a) {
     if (!active) return;
     // D layout of the 32x32 MFMA: register v of lane j holds D[8*(v/4) + 4*(j/32) + v%4][j%32];
     // D rows = my 32 activation rows, D cols = output channels; (re, im) = (K1 - K3, K1 + K2)
-    const int ntw = split ? 1 : NT;
+    const int oc = DH_COLS * ob + 2 * (32 * t0 + cl);
+    if (oc >= a.O2) return;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int nn = r0 + 32 * rb + 8 * (v >> 2) + 4 * kh + (v & 3);
         if (nn >= ncols) continue;
         const int m2 = nn / a.B, b2 = nn - m2 * a.B;
         float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const int oc = DH_COLS * ob + 2 * (32 * (t0 + t) + cl);
-            if (t < ntw && oc < a.O2) *reinterpret_cast<f2*>(orow + oc) = f2{acc[0][t][v] - acc[2][t][v], acc[0][t][v] + acc[1][t][v]};
-        }
+        *reinterpret_cast<f2*>(orow + oc) = f2{acc[0][v] - acc[2][v], acc[0][v] + acc[1][v]};
     }
 }
 
@@ -362,7 +347,7 @@ int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s) {
 int dhconv_launch(const DhconvArgs& a, hipStream_t s) {
     const int64_t rows_max = (int64_t)a.M * a.B;
     if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
-    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
+    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + DH_GROUP - 1) / DH_GROUP));
     const bool vec4 = a.I2 % 4 == 0 && a.ld_in % 4 == 0;
     if (vec4)
         hipLaunchKernelGGL((dhconv_kernel<true>), grid, dim3(256), 0, s, a);

@@ -35,18 +35,19 @@ constexpr int PW_KALIGN = 128;    // K is padded to whole unrolled loop bodies (
 __device__ __forceinline__ float bf16_to_f(unsigned short h) { return __uint_as_float((unsigned int)h << 16); }
 __device__ __forceinline__ unsigned short f_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
 
-// exact (erf) GELU; erf by Abramowitz-Stegun 7.1.26 (|error| < 1.5e-7), written without cancellation in the
-// negative tail: 1 + erf(z) = poly * exp(-z^2) for z < 0 (relative error there stays below 1e-2, at values
-// under 1e-6 in magnitude)
+// exact (erf) GELU; erf by Abramowitz-Stegun 7.1.26 (|error| < 1.5e-7).  With q(z) = poly(t) exp(-z^2) ~ erfc(z),
+// z = |x| / sqrt 2:  gelu(x) = max(x, 0) - |x| q(z) / 2  for both signs, so there is no cancellation in the negative
+// tail (relative error there stays below 1e-2, at values under 1e-6 in magnitude).  Everything is written in
+// u = z sqrt(log2 e), which turns exp(-z^2) into one exp2 of a product.
 __device__ __forceinline__ float gelu(float x) {
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    const float u = fabsf(x) * 0.84932180028801904f;                                  // z sqrt(log2 e)
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.27273748087922250f, u, 1.0f));       // 1 / (1 + 0.3275911 z)
     float p = fmaf(t, 1.061405429f, -1.453152027f);
     p = fmaf(t, p, 1.421413741f);
     p = fmaf(t, p, -0.284496736f);
     p = fmaf(t, p, 0.254829592f);
-    const float pe = p * t * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896341f);
-    return 0.5f * x * (x < 0.f ? pe : 2.0f - pe);
+    const float q = p * t * __builtin_amdgcn_exp2f(-u * u);
+    return fmaf(-0.58870501125773735f * u, q, fmaxf(x, 0.f));                         // |x| / 2 = u / (2 * 0.8493218)
 }
 
 // WM = wavefronts along the output rows: 4 (x 2 along pixels: 384 rows x 128 pixels per workgroup) or

@@ -35,7 +35,7 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, inverse ? 1 : 0, p.csphase);
     std::vector<float> packed;
     std::vector<int64_t> aoff;
-    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.compute == SFNO_COMPUTE_BF16, packed, aoff);
+    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.format, packed, aoff);
     // a workgroup covers two 32-row blocks of each parity
     const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
@@ -53,7 +53,7 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     std::vector<int2> work;
     build_worklist(nrb, cost, work, 2);
     t.n_work = (int)work.size();
-    t.n_blocks = (int64_t)(packed.size() / (p.compute == SFNO_COMPUTE_BF16 ? PG_BLOCK_FLOATS / 2 : PG_BLOCK_FLOATS));
+    t.n_blocks = (int64_t)(packed.size() / pg_block_floats(p.format));
     int rc;
     if ((rc = upload(&t.d_A, packed)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_aoff, aoff)) != SFNO_OK) return rc;
@@ -132,12 +132,14 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if ((directions & SFNO_DIR_INVERSE_ADJOINT) && mmax > nlon / 2 + 1) return SFNO_EUNSUPPORTED;
     if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
     if (!(directions & all_dirs) || (directions & ~all_dirs)) return SFNO_EINVAL;
-    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16) return SFNO_EUNSUPPORTED;
+    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16 && compute != SFNO_COMPUTE_FP32_MFMA) return SFNO_EUNSUPPORTED;
     sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
     if (!p) return SFNO_ENOMEM;
     p->nlat = nlat; p->nlon = nlon; p->lmax = lmax; p->mmax = mmax;
     p->grid = grid; p->norm = norm; p->csphase = csphase ? 1 : 0;
-    p->directions = directions; p->compute = compute;
+    p->directions = directions;
+    p->compute = compute == SFNO_COMPUTE_BF16 ? SFNO_COMPUTE_BF16 : SFNO_COMPUTE_FP32;
+    p->format = compute == SFNO_COMPUTE_BF16 ? PG_FORMAT_BF16 : compute == SFNO_COMPUTE_FP32_MFMA ? PG_FORMAT_FP32 : PG_FORMAT_SPLIT;
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return SFNO_EHIP; }
     std::vector<double> theta(nlat), w(nlat);
     int rc = quadrature(grid, nlat, theta.data(), w.data());
@@ -209,7 +211,7 @@ extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, f
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->fwd, xm, spec, ld);
-    return legendre_fold_launch(true, p->compute == SFNO_COMPUTE_BF16, a, p->fwd.n_work, (hipStream_t)stream);
+    return legendre_fold_launch(true, p->format, a, p->fwd.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec, float* xm, int64_t rows, void* stream) {
@@ -217,7 +219,7 @@ extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv, spec, xm, ld);
-    return legendre_fold_launch(false, p->compute == SFNO_COMPUTE_BF16, a, p->inv.n_work, (hipStream_t)stream);
+    return legendre_fold_launch(false, p->format, a, p->inv.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_sht_analysis(const sfno_sht_plan* p, const void* x, int x_dtype, float* spec, int64_t rows, void* workspace,
@@ -274,7 +276,7 @@ extern "C" int sfno_sht_analysis_adjoint(const sfno_sht_plan* p, const float* gs
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->fwd_adj, gspec, w.xm, ld);
-    int rc = legendre_fold_launch(false, p->compute == SFNO_COMPUTE_BF16, a, p->fwd_adj.n_work, (hipStream_t)stream);
+    int rc = legendre_fold_launch(false, p->format, a, p->fwd_adj.n_work, (hipStream_t)stream);
     if (rc != SFNO_OK) return rc;
     return sfno_irfft(p, w.xm, gx, x_dtype, rows, stream);
 }
@@ -289,7 +291,7 @@ extern "C" int sfno_sht_synthesis_adjoint(const sfno_sht_plan* p, const void* gx
     if (rc != SFNO_OK) return rc;
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv_adj, w.xm, gspec, ld);
-    return legendre_fold_launch(true, p->compute == SFNO_COMPUTE_BF16, a, p->inv_adj.n_work, (hipStream_t)stream);
+    return legendre_fold_launch(true, p->format, a, p->inv_adj.n_work, (hipStream_t)stream);
 }
 
 extern "C" int sfno_sht_forward_adjoint(const sfno_sht_plan* p, const void* gcoeffs, float* gx, int64_t rows, void* workspace,

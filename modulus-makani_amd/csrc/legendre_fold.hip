@@ -19,11 +19,40 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-// BF16: the table stream holds bf16 (8 per lane and chunk: lane (row, kg) has k = 16c + 8kg .. +7) and the
-// contraction runs on v_mfma_f32_32x32x16_bf16 with the panel values rounded to bf16 (nearest even) as they are
-// read from LDS; accumulation stays fp32.
-template <int NT, bool ANALYSIS, bool BF16>
-__global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(PgemmArgs a) {
+// MODE selects the arithmetic of the contraction:
+// LF_FP32:  v_mfma_f32_32x32x2_f32 on the fp32 table stream.
+// LF_BF16:  the table stream holds bf16 (8 per lane and chunk: lane (row, kg) has k = 16c + 8kg .. +7) and the
+//   contraction runs on v_mfma_f32_32x32x16_bf16 with the panel values rounded to bf16 (nearest even) as they are
+//   read from LDS; accumulation stays fp32.
+// LF_SPLIT: fp32 operands on the bf16 matrix pipe.  An fp32 number is exactly the sum of three bf16 numbers (its
+//   24 significant bits cut into 8 + 8 + 8 by truncation), so t * q = sum_ij t_i q_j; the six products with
+//   i + j <= 2 are kept (each dropped one is below 2^-23 of the product, the size of an fp32 rounding), every kept
+//   product is exact in the fp32 accumulator, and one K = 16 step costs 6 x 32 matrix-pipe cycles instead of the
+//   8 x 64 of v_mfma_f32_32x32x2_f32.  The table is split on the host (three bf16 planes in the lane order of
+//   LF_BF16), the panel values as they are read from LDS.  Non-finite inputs turn into NaN (inf - inf).
+enum { LF_FP32 = 0, LF_BF16 = 1, LF_SPLIT = 2 };
+
+// x = hi + mid + lo with 8 significant bits each; the pair (a, b) packed as two bf16 per plane
+__device__ __forceinline__ void split3_pack(float a, float b, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+    const uint32_t ab = __builtin_bit_cast(uint32_t, a), bb = __builtin_bit_cast(uint32_t, b);
+    const float a1 = a - __builtin_bit_cast(float, ab & 0xffff0000u), b1 = b - __builtin_bit_cast(float, bb & 0xffff0000u);
+    const uint32_t a1b = __builtin_bit_cast(uint32_t, a1), b1b = __builtin_bit_cast(uint32_t, b1);
+    const float a2 = a1 - __builtin_bit_cast(float, a1b & 0xffff0000u), b2 = b1 - __builtin_bit_cast(float, b1b & 0xffff0000u);
+    hi = __builtin_amdgcn_perm(bb, ab, 0x07060302u);
+    mid = __builtin_amdgcn_perm(b1b, a1b, 0x07060302u);
+    lo = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b2), __builtin_bit_cast(uint32_t, a2), 0x07060302u);
+}
+
+// resident wavefronts per SIMD: set by the 16 NT accumulator registers and, in split mode, the three-plane fragments
+constexpr int lf_occupancy(int nt, int mode) {
+    if (mode == LF_SPLIT) return nt <= 2 ? 4 : nt <= 4 ? 3 : 2;
+    if (mode == LF_BF16) return nt <= 3 ? 4 : 3;        // the eight gathered panel values per tile need registers too
+    return nt <= 4 ? 4 : 3;
+}
+
+template <int NT, bool ANALYSIS, int MODE>
+__global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_kernel(PgemmArgs a) {
+    constexpr bool BF16 = MODE == LF_BF16;
     constexpr int TN = 32 * NT;
     constexpr int LDQ = TN + ((TN % 64 == 0) ? 32 : 0);
     // [buffer][parity][k][column]; reused for the parity exchange of the synthesis epilogue
@@ -55,7 +84,8 @@ __global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(Pge
     const float* sp_m = (ANALYSIS ? a.Out : a.Q) + (int64_t)m * lmax * ld;     // spectral panel of order m
     // wavefronts without a row block read the head of the table (always at least nc blocks long) and discard it
     // 16 bytes per lane: fp32 blocks are two such pieces per chunk (128 per block), bf16 blocks one (64 per block)
-    constexpr int APB = BF16 ? 64 : 128;
+    constexpr int NA = MODE == LF_BF16 ? 1 : MODE == LF_SPLIT ? 3 : 2;     // 16-byte pieces per lane and block
+    constexpr int APB = 64 * NA;
     const float4* ap = reinterpret_cast<const float4*>(a.A) + ((active ? a.a_off[2 * m + par] + (int64_t)rb * nc : (int64_t)0) * APB + lane);
 
     floatx16 acc[NT];
@@ -117,8 +147,30 @@ __global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(Pge
     const int kh = lane >> 5, cl = lane & 31;
     // One K-chunk of MFMAs.  No branches inside: columns past ld hold zeros in LDS and are
     // masked at the store, so the LDS reads can be issued well ahead of the matrix instructions.
-    auto compute = [&](int buf, const f4 (&ar)[2]) {
-        if constexpr (BF16) {
+    auto compute = [&](int buf, const f4 (&ar)[NA]) {
+        if constexpr (MODE == LF_SPLIT) {
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, ar[0]), a1 = __builtin_bit_cast(bf16x8, ar[1]), a2 = __builtin_bit_cast(bf16x8, ar[2]);
+            const float* qbase = &qs[buf][par][8 * kh][cl];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+                u4 h, mi, lo;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t x, y, z;
+                    split3_pack(qbase[2 * e * LDQ + 32 * t], qbase[(2 * e + 1) * LDQ + 32 * t], x, y, z);
+                    h[e] = x; mi[e] = y; lo[e] = z;
+                }
+                const bf16x8 q0v = __builtin_bit_cast(bf16x8, h), q1v = __builtin_bit_cast(bf16x8, mi), q2v = __builtin_bit_cast(bf16x8, lo);
+                // smallest terms first
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, q0v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q1v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q2v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q0v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q1v, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q0v, acc[t], 0, 0, 0);
+            }
+        } else if constexpr (BF16) {
             // ar[0] carries 8 bf16 table values; every column tile gathers its 8 panel values along k
             const bf16x8 av = __builtin_bit_cast(bf16x8, ar[0]);
             const float* qbase = &qs[buf][par][8 * kh][cl];
@@ -149,16 +201,16 @@ __global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(Pge
         }
     };
     const f4* apv = reinterpret_cast<const f4*>(ap);
-    auto a_load = [&](int c, f4 (&ar)[2]) {
-        ar[0] = apv[(int64_t)c * APB];
-        if (!BF16) ar[1] = apv[(int64_t)c * APB + 64];
+    auto a_load = [&](int c, f4 (&ar)[NA]) {
+#pragma unroll
+        for (int p = 0; p < NA; ++p) ar[p] = apv[(int64_t)c * APB + 64 * p];
     };
 
     // Software pipeline, one chunk deep: the loads of chunk c+1 (raw panel rows and table
     // fragments) are issued before the MFMAs of chunk c and are first touched after them.
     // The explicit wait for all of them at the end of the iteration keeps the wait-count
     // bookkeeping of the next iteration's MFMA block empty.
-    f4 acur[2], anext[2];
+    f4 acur[NA], anext[NA];
     if (nc > 0) {
         q_load(0);
         a_load(0, acur);
@@ -179,8 +231,8 @@ __global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(Pge
         if (more) q_store(buf ^ 1, c + 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): everything issued above has landed
         __syncthreads();
-        acur[0] = anext[0];
-        acur[1] = anext[1];
+#pragma unroll
+        for (int p = 0; p < NA; ++p) acur[p] = anext[p];
     }
 
     // D layout of the 32x32 MFMA: register v of lane j holds D[8*(v/4) + 4*(j/32) + v%4][j%32].
@@ -226,7 +278,7 @@ __global__ __launch_bounds__(256, NT <= 4 ? 4 : 3) void legendre_fold_kernel(Pge
     }
 }
 
-template <bool ANALYSIS, bool BF16>
+template <bool ANALYSIS, int MODE>
 static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     const int64_t ncols = a.ld;
     if (n_work <= 0 || ncols <= 0) return SFNO_OK;
@@ -241,7 +293,7 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
 #define LF_CASE(NT_)                                                                                 \
     case NT_: {                                                                                      \
         dim3 grid(n_work, (unsigned)((ncols + 32 * NT_ - 1) / (32 * NT_)));                          \
-        hipLaunchKernelGGL((legendre_fold_kernel<NT_, ANALYSIS, BF16>), grid, dim3(256), 0, s, a);   \
+        hipLaunchKernelGGL((legendre_fold_kernel<NT_, ANALYSIS, MODE>), grid, dim3(256), 0, s, a);   \
         break;                                                                                       \
     }
     switch (best) {
@@ -252,9 +304,13 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
-int legendre_fold_launch(bool analysis, bool bf16, const PgemmArgs& a, int n_work, hipStream_t s) {
-    if (bf16) return analysis ? launch_fold<true, true>(a, n_work, s) : launch_fold<false, true>(a, n_work, s);
-    return analysis ? launch_fold<true, false>(a, n_work, s) : launch_fold<false, false>(a, n_work, s);
+int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_work, hipStream_t s) {
+    switch (format) {
+        case PG_FORMAT_BF16: return analysis ? launch_fold<true, LF_BF16>(a, n_work, s) : launch_fold<false, LF_BF16>(a, n_work, s);
+        case PG_FORMAT_SPLIT: return analysis ? launch_fold<true, LF_SPLIT>(a, n_work, s) : launch_fold<false, LF_SPLIT>(a, n_work, s);
+        case PG_FORMAT_FP32: return analysis ? launch_fold<true, LF_FP32>(a, n_work, s) : launch_fold<false, LF_FP32>(a, n_work, s);
+    }
+    return SFNO_EINVAL;
 }
 
 }  // namespace sfno

@@ -105,11 +105,16 @@ struct LegendreGen {
 void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work,
                     int rb_step = PG_WAVES);
 // equator-folded Legendre streams (two per order: even and odd l+m), see tables.cpp
-// bf16 = true packs 8 bf16 per lane and chunk (half the bytes; `packed` then holds 256 floats = 1 KiB per block)
+// format of one 32 x 16 block of the stream:
+//   PG_FORMAT_FP32 : 512 floats, fragments of v_mfma_f32_32x32x2_f32
+//   PG_FORMAT_BF16 : 8 bf16 per lane (rounded to nearest even), 256 floats = 1 KiB
+//   PG_FORMAT_SPLIT: three planes of 8 bf16 per lane whose sum is the fp32 value exactly, 768 floats = 3 KiB
+enum { PG_FORMAT_FP32 = 0, PG_FORMAT_BF16 = 1, PG_FORMAT_SPLIT = 2 };
+inline int pg_block_floats(int format) { return format == PG_FORMAT_BF16 ? 256 : format == PG_FORMAT_SPLIT ? 768 : 512; }
 // value = P * lat_w[k] * order_scale[m]; a null pointer stands for all ones
-void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, bool bf16,
+void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
                         std::vector<float>& packed, std::vector<int64_t>& aoff);
-int legendre_fold_launch(bool analysis, bool bf16, const PgemmArgs& a, int n_work, hipStream_t s);
+int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
 struct FftPlan {
@@ -143,6 +148,7 @@ int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, int 
 
 struct sfno_sht_plan {
     int nlat, nlon, lmax, mmax, grid, norm, csphase, directions, compute, device;
+    int format;                         // PG_FORMAT_* of the Legendre streams
     sfno::PgemmTable fwd, inv;          // analysis (forward) and synthesis (inverse) streams
     sfno::PgemmTable fwd_adj, inv_adj;  // their adjoints: synthesis-format stream of the analysis table and vice versa
     sfno::FftPlan fft;

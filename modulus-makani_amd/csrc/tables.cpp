@@ -219,7 +219,33 @@ static void pack_blocks_bf16(unsigned short* dst, int rows, int K, G get) {
         }
 }
 
-void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, bool bf16,
+// three-plane flavour: block = 3 planes x 64 lanes x 8 bf16, same (lane, e) -> (row, k) map as pack_blocks_bf16; the planes
+// hold the fp32 value cut into its upper, middle and lower 8 significant bits (truncation, so the sum is exact)
+template <class G>
+static void pack_blocks_split(unsigned short* dst, int rows, int K, G get) {
+    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
+    for (int rb = 0; rb < nrb; ++rb)
+        for (int c = 0; c < nc; ++c) {
+            unsigned short* blk = dst + ((size_t)rb * nc + c) * 1536;
+            for (int j = 0; j < 64; ++j)
+                for (int e = 0; e < 8; ++e) {
+                    int row = PG_ROWS * rb + (j & 31);
+                    int k = PG_KC * c + 8 * (j >> 5) + e;
+                    float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
+                    for (int pl = 0; pl < 3; ++pl) {
+                        uint32_t u;
+                        std::memcpy(&u, &v, 4);
+                        u &= 0xffff0000u;
+                        float t;
+                        std::memcpy(&t, &u, 4);
+                        blk[(pl * 64 + j) * 8 + e] = (unsigned short)(u >> 16);
+                        v -= t;
+                    }
+                }
+        }
+}
+
+void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
                         std::vector<float>& packed, std::vector<int64_t>& aoff) {
     const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
     const int K2 = (nlat + 1) / 2;
@@ -233,7 +259,7 @@ void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double*
             int64_t nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl_p(m, 0) + PG_KC - 1) / PG_KC;
             tot += nrb * nc;
         }
-    const size_t blk_floats = bf16 ? PG_BLOCK_FLOATS / 2 : PG_BLOCK_FLOATS;
+    const size_t blk_floats = (size_t)pg_block_floats(format);
     packed.assign((size_t)tot * blk_floats, 0.0f);
     float* base = packed.data();
     parallel_for(mmax, [&, base](int m) {
@@ -251,10 +277,13 @@ void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double*
             auto lw = [=](int k) { return lat_w ? lat_w[k] * sc : sc; };
             auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * lw(k); };
             auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] * lw(row) : 0.0; };
-            if (bf16) {
-                unsigned short* d16 = reinterpret_cast<unsigned short*>(dst);
+            unsigned short* d16 = reinterpret_cast<unsigned short*>(dst);
+            if (format == PG_FORMAT_BF16) {
                 if (analysis) pack_blocks_bf16(d16, np, K2, wa);
                 else pack_blocks_bf16(d16, K2, kpad, ws);
+            } else if (format == PG_FORMAT_SPLIT) {
+                if (analysis) pack_blocks_split(d16, np, K2, wa);
+                else pack_blocks_split(d16, K2, kpad, ws);
             } else {
                 if (analysis) pack_blocks(dst, np, K2, wa);
                 else pack_blocks(dst, K2, kpad, ws);

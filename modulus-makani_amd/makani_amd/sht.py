@@ -70,7 +70,7 @@ class _Plan:
             check(
                 lib.sfno_sht_plan_create(
                     mod.nlat, mod.nlon, mod.lmax, mod.mmax, _lib.GRID[mod.grid], _lib.NORM[mod.norm], int(mod.csphase), directions,
-                    _lib.COMPUTE_BF16 if mod.compute == "bf16" else _lib.COMPUTE_FP32, ctypes.byref(self.handle),
+                    {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16, "fp32_mfma": _lib.COMPUTE_FP32_MFMA}[mod.compute], ctypes.byref(self.handle),
                 ),
                 "sfno_sht_plan_create",
             )
@@ -95,9 +95,12 @@ class _SHTBase(nn.Module):
 
     def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, compute="fp32"):
         super().__init__()
-        # compute = "bf16": Legendre stage on bf16 MFMA (bf16 tables and inputs, fp32 accumulation); default and reference: fp32
-        if compute not in ("fp32", "bf16"):
-            raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32' or 'bf16'")
+        # compute = "fp32" (default, the reference's arithmetic): fp32 operands and accumulation, the Legendre stage on the
+        #   bf16 matrix pipe with every operand cut exactly into three bf16 numbers;
+        # "fp32_mfma": the same on the fp32 matrix instruction;
+        # "bf16": bf16 tables and inputs, fp32 accumulation.
+        if compute not in ("fp32", "bf16", "fp32_mfma"):
+            raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32', 'fp32_mfma' or 'bf16'")
         self.compute = compute
         self.nlat = nlat
         self.nlon = nlon

@@ -170,6 +170,40 @@ def test_bf16_compute_variant(lib_built, nlat, nlon, lmax, mmax, grid, lead):
     assert e_fwd > 1e-5 or e_inv > 1e-5          # it is the reduced-precision path that ran
 
 
+@pytest.mark.parametrize("nlat,nlon,lmax,mmax,grid,lead", [CASES[0], CASES[8], CASES[9], (241, 480, 241, 241, "legendre-gauss", (12,))])
+def test_fp32_on_bf16_pipe_is_as_accurate_as_fp32_mfma(lib_built, nlat, nlon, lmax, mmax, grid, lead):
+    """The default fp32 mode cuts every operand of the Legendre stage exactly into three bf16 numbers and keeps the six
+    largest partial products; "fp32_mfma" runs the same contraction on the fp32 matrix instruction.  Both meet the fp32
+    bound against the float64 oracle, and the split path is not less accurate than the plain one (its dropped terms are
+    below one fp32 rounding of a product)."""
+    import makani_amd as ma
+
+    print(f"case fp32 modes {nlat}x{nlon} lmax={lmax} mmax={mmax} {grid} lead={lead}", flush=True)
+    t = ShtTables(nlat, nlon, lmax, mmax, grid)
+    torch.manual_seed(9)
+    # a wide spread of magnitudes and all 24 significant bits in use
+    x = torch.randn(*lead, nlat, nlon) * torch.exp(3.0 * torch.randn(*lead, 1, 1))
+    c = torch.randn(*lead, t.lmax, t.mmax, dtype=torch.complex64) * torch.exp(3.0 * torch.randn(*lead, 1, 1))
+    ref = sht_forward(x.double().numpy(), t)
+    refi = sht_inverse(c.numpy().astype(np.complex128), t)
+    err = {}
+    for mode in ("fp32", "fp32_mfma"):
+        got = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute=mode)(x.cuda())
+        goti = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid=grid, compute=mode)(c.cuda())
+        err[mode] = (rel_l2(got.cpu().numpy(), ref), rel_l2(goti.cpu().numpy(), refi))
+        print(f"   {mode}: rel-L2 forward {err[mode][0]:.2e} inverse {err[mode][1]:.2e}", flush=True)
+        assert err[mode][0] < TOL and err[mode][1] < TOL
+    assert err["fp32"][0] <= 2.0 * err["fp32_mfma"][0] + 1e-7
+    assert err["fp32"][1] <= 2.0 * err["fp32_mfma"][1] + 1e-7
+
+
+def test_unknown_compute_mode_raises(lib_built):
+    import makani_amd as ma
+
+    with pytest.raises(ValueError):
+        ma.RealSHT(8, 16, compute="fp16")
+
+
 def test_known_answers_config0(lib_built):
     """configs[0] (equiangular 32 x 64, lmax 32, mmax 33, batch 2, 4 channels) against the committed known answers
     of tests/golden (scipy spherical harmonics, no oracle involved): rel-L2 <= 1e-5 both ways."""

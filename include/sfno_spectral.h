@@ -212,6 +212,18 @@ size_t sfno_dhconv_workspace_bytes(const sfno_dhconv_weights* w, int batch, int 
 int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y, int batch, int mmax,
                 int triangular, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- per-degree power (spectral losses) ------------------------------------------------ */
+
+/* power[r][l] = |c[r,l,0]|^2 + 2 sum_{0<m<mmax} |c[r,l,m]|^2 from coefficients in the spectral layout (the output of
+ * sfno_sht_analysis): the reduction GeometricH1Loss applies to RealSHT output before it weights the degrees with
+ * l(l+1) (makani/utils/losses.py:301-305, 320-331), without the pass to the reference coefficient layout.
+ * spec: float [mmax][lmax][sfno_spectral_ld(rows)], power: float [rows][lmax]. */
+int sfno_degree_power(const float* spec, float* power, int64_t rows, int lmax, int mmax, void* stream);
+/* cotangent of the above in the spectral layout, ready for sfno_sht_analysis_adjoint:
+ * gspec[r,l,m] = 2 w_m gpower[r][l] c[r,l,m], w_0 = 1, w_m = 2 otherwise */
+int sfno_degree_power_grad(const float* spec, const float* gpower, float* gspec, int64_t rows, int lmax, int mmax,
+                           void* stream);
+
 /* ---- "diagonal" operator ------------------------------------------------------------- */
 
 /* y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l,m] (makani/models/common/contractions.py:121-127, operator_type

@@ -438,6 +438,16 @@ extern "C" int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y,
 
 // ---- diagonal operator -----------------------------------------------------------------------------
 
+extern "C" int sfno_degree_power(const float* spec, float* power, int64_t rows, int lmax, int mmax, void* stream) {
+    if (!spec || !power || !rows_ok(rows)) return SFNO_EINVAL;
+    return degree_power_launch(spec, power, rows, lmax, mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+}
+
+extern "C" int sfno_degree_power_grad(const float* spec, const float* gpower, float* gspec, int64_t rows, int lmax, int mmax, void* stream) {
+    if (!spec || !gpower || !gspec || !rows_ok(rows)) return SFNO_EINVAL;
+    return degree_power_grad_launch(spec, gpower, gspec, rows, lmax, mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
+}
+
 extern "C" int sfno_diagonal_contract(const void* x, const void* weight, void* y, int batch, int in_channels, int out_channels,
                                       int64_t positions, int adjoint, void* stream) {
     if (!x || !weight || !y || batch < 1 || in_channels < 1 || out_channels < 1 || positions < 1) return SFNO_EINVAL;

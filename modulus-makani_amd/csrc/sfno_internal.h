@@ -137,6 +137,10 @@ int rfft_launch(const FftPlan& p, const void* x, int x_dtype, float* xm, int64_t
 // xm [mmax][nlat][ld] -> x [rows][nlat][nlon]
 int irfft_launch(const FftPlan& p, const float* xm, void* x, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
 
+// ---- per-degree power of spectral-layout coefficients and its gradient (degree_power.hip) ------------
+int degree_power_launch(const float* spec, float* power, int64_t rows, int lmax, int mmax, int ld, hipStream_t s);
+int degree_power_grad_launch(const float* spec, const float* gpower, float* gspec, int64_t rows, int lmax, int mmax, int ld, hipStream_t s);
+
 // ---- layout passes (layout.hip) ----------------------------------------------------------
 int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri,
                               hipStream_t s);

@@ -66,6 +66,8 @@ def _load():
         "sfno_dhconv_spectral": (i32, [vp, vp, vp, i32, i32, i32, vp]),
         "sfno_dhconv_workspace_bytes": (sz, [vp, i32, i32]),
         "sfno_dhconv": (i32, [vp, vp, vp, i32, i32, i32, vp, sz, vp]),
+        "sfno_degree_power": (i32, [vp, vp, i64, i32, i32, vp]),
+        "sfno_degree_power_grad": (i32, [vp, vp, vp, i64, i32, i32, vp]),
         "sfno_diagonal_contract": (i32, [vp, vp, vp, i32, i32, i32, i64, i32, vp]),
         "sfno_diagonal_weight_grad": (i32, [vp, vp, vp, i32, i32, i32, i64, vp]),
         "sfno_pointwise_weight_elems": (i64, [i32, i32]),

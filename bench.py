@@ -212,6 +212,10 @@ def bench_sht_pair(args):
             "traffic": read_traffic(dom),
             "algorithmic_flops_per_launch": leg_flops,
             "avg_launch_ms": stage_ms[dom],
+            "note": ("algorithmic (triangular) fp32 flops over the kernel's time, priced against the fp32 matrix peak; the kernel "
+                     "executes half of those MACs (equator fold)"
+                     + (" and forms every fp32 product from six bf16 MFMA partial products of exactly split operands" if args.compute == "fp32"
+                        else " on bf16 MFMA")),
         },
         "stages_ms": stage_ms,
         "fft_hbm": {

@@ -45,8 +45,7 @@ __device__ __forceinline__ void split3_pack(float a, float b, uint32_t& hi, uint
 
 // resident wavefronts per SIMD: set by the 16 NT accumulator registers and, in split mode, the three-plane fragments
 constexpr int lf_occupancy(int nt, int mode) {
-    if (mode == LF_SPLIT) return nt <= 2 ? 4 : nt <= 4 ? 3 : 2;
-    if (mode == LF_BF16) return nt <= 3 ? 4 : 3;        // the eight gathered panel values per tile need registers too
+    if (mode == LF_SPLIT) return nt <= 3 ? 4 : 3;
     return nt <= 4 ? 4 : 3;
 }
 
@@ -100,6 +99,9 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
     // Loads are unconditional (indices clamped into the panel) and keep the raw rows in
     // registers; masking and the mirror sum/difference happen when the chunk is written to
     // LDS, one chunk of MFMAs later.
+    // uniform panel base + 32-bit byte offset per lane (a panel is far smaller than 4 GiB): one address register per load
+    const char* qpanel = reinterpret_cast<const char*>(ANALYSIS ? xm_m : sp_m);
+    auto q_at = [&](int row, int n) { return *reinterpret_cast<const f4*>(qpanel + (size_t)(((uint32_t)row * (uint32_t)ld + (uint32_t)n) * 4u)); };
     auto q_load = [&](int c) {
 #pragma unroll
         for (int u = 0; u < QV; ++u) {
@@ -108,12 +110,11 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
             const int i = c * PG_KC + row, n = min(n0 + 4 * c4, ld - 4);
             if (ANALYSIS) {
                 const int k = min(i, K2 - 1);
-                q0[u] = *reinterpret_cast<const f4*>(xm_m + (int64_t)k * ld + n);
-                q1[u] = *reinterpret_cast<const f4*>(xm_m + (int64_t)(nlat - 1 - k) * ld + n);
+                q0[u] = q_at(k, n);
+                q1[u] = q_at(nlat - 1 - k, n);
             } else {
-                const int l0 = min(m + 2 * i, lmax - 1), l1 = min(m + 2 * i + 1, lmax - 1);
-                q0[u] = *reinterpret_cast<const f4*>(sp_m + (int64_t)l0 * ld + n);
-                q1[u] = *reinterpret_cast<const f4*>(sp_m + (int64_t)l1 * ld + n);
+                q0[u] = q_at(min(m + 2 * i, lmax - 1), n);
+                q1[u] = q_at(min(m + 2 * i + 1, lmax - 1), n);
             }
         }
     };
@@ -169,6 +170,8 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
                 acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q0v, acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q1v, acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q0v, acc[t], 0, 0, 0);
+                // one tile at a time: the split values of several tiles in flight would not fit the registers
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else if constexpr (BF16) {
             // ar[0] carries 8 bf16 table values; every column tile gathers its 8 panel values along k

@@ -65,10 +65,11 @@ extern "C" {
 #define SFNO_DTYPE_BF16 1
 
 /* arithmetic of the Legendre / channel-mix contractions */
-#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  The Legendre stage runs them on the bf16 matrix
-                                  * pipe: each operand is cut exactly into three bf16 numbers and the six products
-                                  * larger than 2^-23 of the result are accumulated in fp32 (error of the size of
-                                  * fp32 rounding); the channel mix runs on fp32 MFMA. */
+#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  The Legendre stage and the channel mix run them on
+                                  * the bf16 matrix pipe: each operand is cut exactly into three bf16 numbers and the
+                                  * six products larger than 2^-23 of the result are accumulated in fp32 (error of the
+                                  * size of fp32 rounding).  Channel mixes with an odd number of input channels run
+                                  * on fp32 MFMA. */
 #define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs (tables and activations rounded to bf16), fp32 accumulate */
 #define SFNO_COMPUTE_FP32_MFMA 2 /* transform plans only: as SFNO_COMPUTE_FP32 with the Legendre stage on the fp32 MFMA
                                   * instruction (fp32 tables, no operand splitting) */

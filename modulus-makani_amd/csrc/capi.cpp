@@ -342,9 +342,15 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
     sfno_dhconv_weights* w = new (std::nothrow) sfno_dhconv_weights();
     if (!w) return SFNO_ENOMEM;
     w->I = I; w->O = O; w->L = L; w->compute = compute;
+    // fp32 on the bf16 matrix pipe reads activation rows in groups of four floats; odd channel counts stay on fp32 MFMA
+    w->split = compute == SFNO_COMPUTE_FP32 && (2 * I) % 4 == 0;
     if (hipGetDevice(&w->device) != hipSuccess) { delete w; return SFNO_EHIP; }
     size_t bytes;
-    if (compute == SFNO_COMPUTE_BF16) {
+    if (w->split) {
+        w->nob = (2 * O + 127) / 128;
+        w->nc = (2 * I + 15) / 16;
+        bytes = 6144 * (size_t)L * w->nob * w->nc;          // 3 planes x 64 x 8 complex bf16 per (degree, column block, chunk)
+    } else if (compute == SFNO_COMPUTE_BF16) {
         w->nob = (2 * O + 255) / 256;
         w->nc = (2 * I + 31) / 32;
         bytes = 8192 * (size_t)L * w->nob * w->nc;          // 128 x 16 complex bf16 per (degree, column block, chunk)
@@ -360,6 +366,8 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
 
 static int pack_weights(sfno_dhconv_weights* w, const void* weight, int adjoint, void* stream) {
     if (!w || !weight) return SFNO_EINVAL;
+    if (w->split)
+        return dhconv_pack_split_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
     if (w->compute == SFNO_COMPUTE_BF16)
         return dhconv_pack_bf16_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
     return dhconv_pack_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
@@ -411,6 +419,7 @@ extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* s
     a.ld_out = (int)sfno_spectral_ld((int64_t)batch * w->O);
     a.nob = w->nob;
     a.nc = w->nc;
+    if (w->split) return dhconv_split_launch(a, (hipStream_t)stream);
     if (w->compute == SFNO_COMPUTE_BF16) return dhconv_bf16_launch(a, (hipStream_t)stream);
     return dhconv_launch(a, (hipStream_t)stream);
 }

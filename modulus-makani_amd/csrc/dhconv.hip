@@ -186,6 +186,7 @@ int dhconv_pack_launch(const float2* w, float* packed, int I, int O, int L, int 
 // contiguous bytes of its activation row and 16 contiguous bytes of a weight column per step.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 constexpr int DHB_COLS = 256;          // output columns o' per workgroup
 constexpr int DHB_KC = 32;             // i' per chunk
 
@@ -341,6 +342,201 @@ int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s) {
     if (a.I2 % 4 != 0 || a.ld_in % 4 != 0) return SFNO_EUNSUPPORTED;
     dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
     hipLaunchKernelGGL(dhconv_bf16_kernel, grid, dim3(256), 0, s, a);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+// ---- fp32 on the bf16 matrix pipe -----------------------------------------------------------------------
+// The decomposition of dhconv_bf16_kernel (2x2 real embedding, activation rows as A operands straight from the
+// spectral layout, weights expanded into LDS) with fp32 accuracy: every operand is cut exactly into three bf16
+// numbers (8 + 8 + 8 significant bits, by truncation) and the six partial products larger than 2^-23 of the result are
+// accumulated in fp32, each of them exact.  One K = 16 step then costs 6 x 32 matrix-pipe cycles; the fp32 instruction
+// needs 8 x 64 for the four real products of the embedding and 6 x 64 for Gauss's three.  The weights are stored as
+// three planes of complex bf16 (12 bytes per complex weight), split when they are packed; the activations are split in
+// registers, once per 16 values and wavefront, and reused for the four column tiles.
+constexpr int DHS_COLS = 128;          // output columns o' per workgroup
+constexpr int DHS_KC = 16;             // i' per chunk: one matrix K step, small enough for four workgroups per CU
+
+// x = hi + mid + lo with 8 significant bits each; the pair (a, b) packed as two bf16 per plane
+__device__ __forceinline__ void dh_split3(float a, float b, unsigned int& hi, unsigned int& mid, unsigned int& lo) {
+    const unsigned int ab = __builtin_bit_cast(unsigned int, a), bb = __builtin_bit_cast(unsigned int, b);
+    const float a1 = a - __builtin_bit_cast(float, ab & 0xffff0000u), b1 = b - __builtin_bit_cast(float, bb & 0xffff0000u);
+    const unsigned int a1b = __builtin_bit_cast(unsigned int, a1), b1b = __builtin_bit_cast(unsigned int, b1);
+    const float a2 = a1 - __builtin_bit_cast(float, a1b & 0xffff0000u), b2 = b1 - __builtin_bit_cast(float, b1b & 0xffff0000u);
+    hi = __builtin_amdgcn_perm(bb, ab, 0x07060302u);
+    mid = __builtin_amdgcn_perm(b1b, a1b, 0x07060302u);
+    lo = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned int, b2), __builtin_bit_cast(unsigned int, a2), 0x07060302u);
+}
+
+// grid = (8 * ceil(L/8) * nob, row groups of 128), nob = ceil(2*O / 128); requires 2*I % 4 == 0
+__global__ __launch_bounds__(256, 4) void dhconv_split_kernel(DhconvArgs a) {
+    constexpr int NT = DHS_COLS / 32;                // 4 column tiles per wavefront
+    constexpr int PITCH = DHS_KC + 8;                // bf16 elements per LDS row (48 bytes: 16-byte reads of 8 lanes hit distinct banks)
+    constexpr int PLANE = DHS_COLS * PITCH;
+    __shared__ __align__(16) unsigned short ws[2][3][DHS_COLS][PITCH];
+
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
+    if (lidx >= a.L) return;
+    const int l = a.L - 1 - lidx;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
+    const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;
+    const int r0 = blockIdx.y * 128;
+    if (r0 >= ncols) return;
+    const bool active = r0 + 32 * wave < ncols;
+    const int nc = a.nc;                                           // chunks of 16 i'
+    const int kg = lane >> 5, cl = lane & 31;
+
+    const int n = min(r0 + 32 * wave + cl, ncols - 1);
+    const int mm = n / a.B, bb = n - mm * a.B;
+    const float* xrow = a.X + ((int64_t)mm * a.L + l) * a.ld_in + (int64_t)bb * a.I2;
+    // packed weights of (l, ob): nc chunks of 3 planes x 64 (o) x 8 (i) complex bf16 = 6 KiB, one 8-byte piece per thread and plane
+    const u2* wp = reinterpret_cast<const u2*>(a.W) + ((int64_t)l * a.nob + ob) * nc * 768 + tid;
+
+    floatx16 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+
+    // my 8 activations of the chunk: i' = 16c + 8kg .. +7 (clamped in groups of four; weights are zero past 2*I)
+    auto x_load = [&](int c, f4 (&xr)[2]) {
+        const int k = DHS_KC * c + 8 * kg;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) xr[j] = *reinterpret_cast<const f4*>(xrow + min(k + 4 * j, a.I2 - 4));
+    };
+    auto w_load = [&](int c, u2 (&w)[3]) {
+#pragma unroll
+        for (int p = 0; p < 3; ++p) w[p] = wp[(int64_t)c * 768 + 256 * p];
+    };
+    // piece tid (8 bytes = 2 complex = 4 i') of a plane: o = tid / 4, i-group g = tid % 4; it becomes 8 bytes of row 2o
+    // (re, -im, ...) and 8 bytes of row 2o+1 (im, re, ...); negating a number negates each of its three parts
+    auto w_store = [&](int buf, const u2 (&w)[3]) {
+        const int o = tid >> 2, g = tid & 3;
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            const u2 even = w[p] ^ 0x80000000u;
+            const u2 odd = (w[p] >> 16) | (w[p] << 16);
+            *reinterpret_cast<u2*>(&ws[buf][p][2 * o][4 * g]) = even;
+            *reinterpret_cast<u2*>(&ws[buf][p][2 * o + 1][4 * g]) = odd;
+        }
+    };
+    auto compute = [&](int buf, const f4 (&xr)[2]) {
+        {
+            u4 h, mi, lo;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const f4 src = xr[e >> 1];
+                unsigned int x, y, z;
+                dh_split3(src[2 * (e & 1)], src[2 * (e & 1) + 1], x, y, z);
+                h[e] = x; mi[e] = y; lo[e] = z;
+            }
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, h), a1 = __builtin_bit_cast(bf16x8, mi), a2 = __builtin_bit_cast(bf16x8, lo);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const unsigned short* wb = &ws[buf][0][32 * t + cl][8 * kg];
+                const bf16x8 b0 = *reinterpret_cast<const bf16x8*>(wb), b1 = *reinterpret_cast<const bf16x8*>(wb + PLANE),
+                             b2 = *reinterpret_cast<const bf16x8*>(wb + 2 * PLANE);
+                // smallest terms first
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, b0, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b2, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[t], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);       // one tile's fragments in registers at a time
+            }
+        }
+    };
+
+    f4 xcur[2], xnext[2];
+    u2 wnext[3];
+    x_load(0, xcur);
+    w_load(0, wnext);
+    w_store(0, wnext);
+    __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0)
+    __syncthreads();
+    for (int c = 0; c < nc; ++c) {
+        const int buf = c & 1;
+        const bool more = c + 1 < nc;
+        if (more) {
+            w_load(c + 1, wnext);
+            x_load(c + 1, xnext);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (active) compute(buf, xcur);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) w_store(buf ^ 1, wnext);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        xcur[0] = xnext[0];
+        xcur[1] = xnext[1];
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int nn = r0 + 32 * wave + 8 * (v >> 2) + 4 * kg + (v & 3);
+        if (nn >= ncols) continue;
+        const int m2 = nn / a.B, b2 = nn - m2 * a.B;
+        float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int oc = DHS_COLS * ob + 32 * t + cl;
+            if (oc < a.O2) orow[oc] = acc[t][v];
+        }
+    }
+}
+
+// packed[l][ob][c][plane][o (64)][i (8)] = bf16(re part) | bf16(im part) << 16 of plane `plane` of w[8c + i][64 ob + o][l], zero
+// outside the weight (adjoint: of conj(w[64 ob + o][8c + i][l]), w being [O][I][L]); plane p of a float is its p-th group of 8
+// significant bits
+__global__ __launch_bounds__(256) void dhconv_pack_split_kernel(const float2* __restrict__ w, unsigned int* __restrict__ packed, int I, int O, int L,
+                                                                int nob, int nc, int adjoint) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)L * nob * nc * 1536;
+    if (idx >= total) return;
+    const int ii = (int)(idx & 7), o = (int)((idx >> 3) & 63);
+    int64_t rem = idx >> 9;
+    const int plane = (int)(rem % 3);
+    rem /= 3;
+    const int c = (int)(rem % nc);
+    rem /= nc;
+    const int ob = (int)(rem % nob), l = (int)(rem / nob);
+    const int i = 8 * c + ii, oo = 64 * ob + o;
+    unsigned int v = 0;
+    if (i < I && oo < O) {
+        float2 z;
+        if (adjoint) {
+            z = w[((int64_t)oo * I + i) * L + l];
+            z.y = -z.y;
+        } else {
+            z = w[((int64_t)i * O + oo) * L + l];
+        }
+        for (int p = 0; p < plane; ++p) {
+            z.x -= __builtin_bit_cast(float, __builtin_bit_cast(unsigned int, z.x) & 0xffff0000u);
+            z.y -= __builtin_bit_cast(float, __builtin_bit_cast(unsigned int, z.y) & 0xffff0000u);
+        }
+        v = (__builtin_bit_cast(unsigned int, z.x) >> 16) | (__builtin_bit_cast(unsigned int, z.y) & 0xffff0000u);
+    }
+    packed[idx] = v;
+}
+
+int dhconv_pack_split_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s) {
+    const int nob = (2 * O + DHS_COLS - 1) / DHS_COLS, nc = (2 * I + DHS_KC - 1) / DHS_KC;
+    const int64_t total = (int64_t)L * nob * nc * 1536;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_pack_split_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc, adjoint);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+int dhconv_split_launch(const DhconvArgs& a, hipStream_t s) {
+    const int64_t rows_max = (int64_t)a.M * a.B;
+    if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
+    if (a.I2 % 4 != 0 || a.ld_in % 4 != 0) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
+    hipLaunchKernelGGL(dhconv_split_kernel, grid, dim3(256), 0, s, a);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

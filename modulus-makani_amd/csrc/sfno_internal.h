@@ -51,6 +51,10 @@ struct DhconvArgs {
 int dhconv_launch(const DhconvArgs& a, hipStream_t s);
 // bf16 MFMA variant: 256 output columns per workgroup, K chunks of 32, weights packed as complex bf16
 int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s);
+// fp32 operands on the bf16 matrix pipe: 128 output columns per workgroup, K chunks of 32, weights packed as three planes of
+// complex bf16 whose sum is the fp32 weight
+int dhconv_split_launch(const DhconvArgs& a, hipStream_t s);
+int dhconv_pack_split_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s);
 // adjoint = 1 packs the conjugate transpose: w then has shape [O][I][L] and element (i, o) is conj(w[o][i])
 int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s);
 // gradient of the contraction with respect to its weight:
@@ -160,6 +164,7 @@ struct sfno_sht_plan {
 
 struct sfno_dhconv_weights {
     int I, O, L, compute, device;
+    int split;                     // fp32 compute with the weights stored as three bf16 planes (even in_channels)
     int nob, nc;                   // column blocks (over 2*O) and K chunks (over 2*I) per degree
     float* d_W = nullptr;          // packed complex weights
 };

@@ -367,8 +367,13 @@ __device__ __forceinline__ void dh_split3(float a, float b, unsigned int& hi, un
     lo = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned int, b2), __builtin_bit_cast(unsigned int, a2), 0x07060302u);
 }
 
+// Matrix and vector instructions of one wavefront overlap only where they alternate in its instruction stream (a
+// wavefront queueing matrix instructions back to back also holds up the vector instructions of the other wavefronts of
+// its SIMD), so the kernel is software-pipelined by hand: while the 24 matrix instructions of chunk c are issued, the
+// activations of chunk c+1 are split and the weights of chunk c+1 are expanded into the other LDS buffer, a few vector
+// instructions after each matrix instruction, behind scheduling fences; the loads run two chunks ahead.
 // grid = (8 * ceil(L/8) * nob, row groups of 128), nob = ceil(2*O / 128); requires 2*I % 4 == 0
-__global__ __launch_bounds__(256, 4) void dhconv_split_kernel(DhconvArgs a) {
+__global__ __launch_bounds__(256, 3) void dhconv_split_kernel(DhconvArgs a) {
     constexpr int NT = DHS_COLS / 32;                // 4 column tiles per wavefront
     constexpr int PITCH = DHS_KC + 8;                // bf16 elements per LDS row (48 bytes: 16-byte reads of 8 lanes hit distinct banks)
     constexpr int PLANE = DHS_COLS * PITCH;
@@ -411,67 +416,111 @@ __global__ __launch_bounds__(256, 4) void dhconv_split_kernel(DhconvArgs a) {
     };
     // piece tid (8 bytes = 2 complex = 4 i') of a plane: o = tid / 4, i-group g = tid % 4; it becomes 8 bytes of row 2o
     // (re, -im, ...) and 8 bytes of row 2o+1 (im, re, ...); negating a number negates each of its three parts
-    auto w_store = [&](int buf, const u2 (&w)[3]) {
-        const int o = tid >> 2, g = tid & 3;
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            const u2 even = w[p] ^ 0x80000000u;
-            const u2 odd = (w[p] >> 16) | (w[p] << 16);
-            *reinterpret_cast<u2*>(&ws[buf][p][2 * o][4 * g]) = even;
-            *reinterpret_cast<u2*>(&ws[buf][p][2 * o + 1][4 * g]) = odd;
+    const int wo_ = tid >> 2, wg_ = tid & 3;
+    auto w_store_even = [&](int buf, int p, const u2 w) { *reinterpret_cast<u2*>(&ws[buf][p][2 * wo_][4 * wg_]) = w ^ 0x80000000u; };
+    auto w_store_odd = [&](int buf, int p, const u2 w) { *reinterpret_cast<u2*>(&ws[buf][p][2 * wo_ + 1][4 * wg_]) = (w >> 16) | (w << 16); };
+    // the three bf16 planes of my 8 activations: pl[0] = upper, pl[1] = middle, pl[2] = lower 8 significant bits
+    auto split_pair = [&](const f4 (&xr)[2], int e, int stage, u4 (&pl)[3], float (&r)[2]) {
+        const f4 src = xr[e >> 1];
+        const float xa = src[2 * (e & 1)], xb = src[2 * (e & 1) + 1];
+        if (stage == 0) {
+            const unsigned int ab = __builtin_bit_cast(unsigned int, xa), bb2 = __builtin_bit_cast(unsigned int, xb);
+            r[0] = xa - __builtin_bit_cast(float, ab & 0xffff0000u);
+            r[1] = xb - __builtin_bit_cast(float, bb2 & 0xffff0000u);
+            pl[0][e] = __builtin_amdgcn_perm(bb2, ab, 0x07060302u);
+        } else {
+            const unsigned int ab = __builtin_bit_cast(unsigned int, r[0]), bb2 = __builtin_bit_cast(unsigned int, r[1]);
+            const float a2 = r[0] - __builtin_bit_cast(float, ab & 0xffff0000u), b2 = r[1] - __builtin_bit_cast(float, bb2 & 0xffff0000u);
+            pl[1][e] = __builtin_amdgcn_perm(bb2, ab, 0x07060302u);
+            pl[2][e] = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned int, b2), __builtin_bit_cast(unsigned int, a2), 0x07060302u);
         }
     };
-    auto compute = [&](int buf, const f4 (&xr)[2]) {
-        {
-            u4 h, mi, lo;
+    auto split_all = [&](const f4 (&xr)[2], u4 (&pl)[3]) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const f4 src = xr[e >> 1];
-                unsigned int x, y, z;
-                dh_split3(src[2 * (e & 1)], src[2 * (e & 1) + 1], x, y, z);
-                h[e] = x; mi[e] = y; lo[e] = z;
-            }
-            const bf16x8 a0 = __builtin_bit_cast(bf16x8, h), a1 = __builtin_bit_cast(bf16x8, mi), a2 = __builtin_bit_cast(bf16x8, lo);
+        for (int e = 0; e < 4; ++e) {
+            float r[2];
+            split_pair(xr, e, 0, pl, r);
+            split_pair(xr, e, 1, pl, r);
+        }
+    };
+    // Chunk `buf` contracted with planes pc; meanwhile xn (chunk c+1) is split into pn and wn (chunk c+1) goes to LDS.
+    // 14 staging steps are dealt out behind the 24 matrix instructions.
+    auto fused = [&](int buf, const u4 (&pc)[3], const f4 (&xn)[2], u4 (&pn)[3], const u2 (&wn)[3]) {
+        const bf16x8 a0 = __builtin_bit_cast(bf16x8, pc[0]), a1 = __builtin_bit_cast(bf16x8, pc[1]), a2 = __builtin_bit_cast(bf16x8, pc[2]);
+        const unsigned short* wb = &ws[buf][0][cl][8 * kg];
+        float r[2];
+        auto step = [&](int sidx) {
+            if (sidx < 8) split_pair(xn, sidx >> 1, sidx & 1, pn, r);
+            else if (sidx < 11) w_store_even(buf ^ 1, sidx - 8, wn[sidx - 8]);
+            else w_store_odd(buf ^ 1, sidx - 11, wn[sidx - 11]);
+        };
+        constexpr int NM = 6 * NT, NS = 14;
+        u4 bq[2][3];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const unsigned short* wb = &ws[buf][0][32 * t + cl][8 * kg];
-                const bf16x8 b0 = *reinterpret_cast<const bf16x8*>(wb), b1 = *reinterpret_cast<const bf16x8*>(wb + PLANE),
-                             b2 = *reinterpret_cast<const bf16x8*>(wb + 2 * PLANE);
-                // smallest terms first
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, b0, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b2, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[t], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);       // one tile's fragments in registers at a time
+        for (int p = 0; p < 3; ++p) bq[0][p] = *reinterpret_cast<const u4*>(wb + p * PLANE);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (t + 1 < NT) {
+#pragma unroll
+                for (int p = 0; p < 3; ++p) bq[(t + 1) & 1][p] = *reinterpret_cast<const u4*>(wb + p * PLANE + 32 * (t + 1) * PITCH);
             }
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, bq[t & 1][0]), b1 = __builtin_bit_cast(bf16x8, bq[t & 1][1]),
+                         b2 = __builtin_bit_cast(bf16x8, bq[t & 1][2]);
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                // smallest terms first: a2 b0, a1 b1, a0 b2, a1 b0, a0 b1, a0 b0
+                const bf16x8 av = (j == 0) ? a2 : (j == 1 || j == 3) ? a1 : a0;
+                const bf16x8 bv = (j == 0 || j == 3 || j == 5) ? b0 : (j == 1 || j == 4) ? b1 : b2;
+                __builtin_amdgcn_sched_barrier(0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[t], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                const int mi = 6 * t + j;
+#pragma unroll
+                for (int sidx = (mi * NS) / NM; sidx < ((mi + 1) * NS) / NM; ++sidx) step(sidx);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // a wavefront without rows still stages its share of the weights
+    auto stage_only = [&](int buf, const u2 (&wn)[3]) {
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            w_store_even(buf ^ 1, p, wn[p]);
+            w_store_odd(buf ^ 1, p, wn[p]);
         }
     };
 
-    f4 xcur[2], xnext[2];
-    u2 wnext[3];
-    x_load(0, xcur);
-    w_load(0, wnext);
-    w_store(0, wnext);
-    __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0)
+    // Register sets alternate between even and odd chunks (no copies: a copy would wait for the load it copies):
+    // iteration c contracts planes P[c & 1], splits X[(c + 1) & 1] into P[(c + 1) & 1], stores W[(c + 1) & 1] to LDS and
+    // then requests chunk c + 3 into those two sets; chunk c + 2 is already on its way into X[c & 1] and W[c & 1].
+    f4 X0[2], X1[2];
+    u2 W0[3], W1[3];
+    u4 P0[3], P1[3];
+    x_load(0, X0);
+    w_load(0, W0);
+    x_load(min(1, nc - 1), X1);
+    w_load(min(1, nc - 1), W1);
+    stage_only(1, W0);                            // chunk 0 into buffer 0
+    split_all(X0, P0);
     __syncthreads();
-    for (int c = 0; c < nc; ++c) {
-        const int buf = c & 1;
-        const bool more = c + 1 < nc;
-        if (more) {
-            w_load(c + 1, wnext);
-            x_load(c + 1, xnext);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (active) compute(buf, xcur);
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) w_store(buf ^ 1, wnext);
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+    auto iter = [&](int c, const u4 (&pc)[3], u4 (&pn)[3], f4 (&xn)[2], u2 (&wn)[3]) {
+        // chunk c+1 is staged even in the last iteration (a repeat of the last chunk, into the idle buffer)
+        if (active) fused(c & 1, pc, xn, pn, wn);
+        else stage_only(c & 1, wn);
+        // xn and wn are consumed: chunk c+3 goes there (chunk c+2 is in flight or has landed in the other sets)
+        x_load(min(c + 3, nc - 1), xn);
+        w_load(min(c + 3, nc - 1), wn);
         __syncthreads();
-        xcur[0] = xnext[0];
-        xcur[1] = xnext[1];
+    };
+    // X0/W0 held chunk 0 (consumed by the prologue): chunk 2 goes there before the loop
+    x_load(min(2, nc - 1), X0);
+    w_load(min(2, nc - 1), W0);
+    int c = 0;
+    for (; c + 1 < nc; c += 2) {
+        iter(c, P0, P1, X1, W1);
+        iter(c + 1, P1, P0, X0, W0);
     }
+    if (c < nc) iter(c, P0, P1, X1, W1);
 
     if (!active) return;
 #pragma unroll

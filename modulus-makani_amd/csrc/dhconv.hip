@@ -539,44 +539,57 @@ __global__ __launch_bounds__(256, 3) void dhconv_split_kernel(DhconvArgs a) {
 
 // packed[l][ob][c][plane][o (64)][i (8)] = bf16(re part) | bf16(im part) << 16 of plane `plane` of w[8c + i][64 ob + o][l], zero
 // outside the weight (adjoint: of conj(w[64 ob + o][8c + i][l]), w being [O][I][L]); plane p of a float is its p-th group of 8
-// significant bits
+// significant bits.  The parameter has l fastest, the stream has it slowest: a workgroup moves the 8 x 64 channel pairs of
+// one (c, ob) for 8 degrees through LDS, reading 64 contiguous bytes per pair and writing 2 KiB contiguous per plane and degree.
+// grid (nc * nob, ceil(L / 8)), block 256
 __global__ __launch_bounds__(256) void dhconv_pack_split_kernel(const float2* __restrict__ w, unsigned int* __restrict__ packed, int I, int O, int L,
                                                                 int nob, int nc, int adjoint) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t total = (int64_t)L * nob * nc * 1536;
-    if (idx >= total) return;
-    const int ii = (int)(idx & 7), o = (int)((idx >> 3) & 63);
-    int64_t rem = idx >> 9;
-    const int plane = (int)(rem % 3);
-    rem /= 3;
-    const int c = (int)(rem % nc);
-    rem /= nc;
-    const int ob = (int)(rem % nob), l = (int)(rem / nob);
-    const int i = 8 * c + ii, oo = 64 * ob + o;
-    unsigned int v = 0;
-    if (i < I && oo < O) {
-        float2 z;
-        if (adjoint) {
-            z = w[((int64_t)oo * I + i) * L + l];
-            z.y = -z.y;
-        } else {
-            z = w[((int64_t)i * O + oo) * L + l];
+    __shared__ float2 tile[512][9];                  // [pair = ii * 64 + o][degree], padded
+    const int c = blockIdx.x % nc, ob = blockIdx.x / nc;
+    const int l0 = blockIdx.y * 8;
+    const int tid = threadIdx.x, dl = tid & 7;
+#pragma unroll 4
+    for (int pass = 0; pass < 16; ++pass) {
+        const int pr = pass * 32 + (tid >> 3);       // eight lanes per pair: one 64-byte segment
+        const int ii = pr >> 6, o = pr & 63;
+        const int i = 8 * c + ii, oo = 64 * ob + o, l = l0 + dl;
+        float2 z = make_float2(0.f, 0.f);
+        if (i < I && oo < O && l < L) {
+            if (adjoint) {
+                z = w[((int64_t)oo * I + i) * L + l];
+                z.y = -z.y;
+            } else {
+                z = w[((int64_t)i * O + oo) * L + l];
+            }
         }
-        for (int p = 0; p < plane; ++p) {
-            z.x -= __builtin_bit_cast(float, __builtin_bit_cast(unsigned int, z.x) & 0xffff0000u);
-            z.y -= __builtin_bit_cast(float, __builtin_bit_cast(unsigned int, z.y) & 0xffff0000u);
-        }
-        v = (__builtin_bit_cast(unsigned int, z.x) >> 16) | (__builtin_bit_cast(unsigned int, z.y) & 0xffff0000u);
+        tile[pr][dl] = z;
     }
-    packed[idx] = v;
+    __syncthreads();
+    for (int d = 0; d < 8; ++d) {
+        const int l = l0 + d;
+        if (l >= L) break;
+        unsigned int* dst = packed + (((int64_t)l * nob + ob) * nc + c) * 1536;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int word = tid + 256 * u;          // o * 8 + ii
+            const int o = word >> 3, ii = word & 7;
+            float2 z = tile[ii * 64 + o][d];
+#pragma unroll
+            for (int plane = 0; plane < 3; ++plane) {
+                const unsigned int xb = __builtin_bit_cast(unsigned int, z.x) & 0xffff0000u, yb = __builtin_bit_cast(unsigned int, z.y) & 0xffff0000u;
+                dst[plane * 512 + word] = (xb >> 16) | yb;
+                z.x -= __builtin_bit_cast(float, xb);
+                z.y -= __builtin_bit_cast(float, yb);
+            }
+        }
+    }
 }
 
 int dhconv_pack_split_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s) {
     const int nob = (2 * O + DHS_COLS - 1) / DHS_COLS, nc = (2 * I + DHS_KC - 1) / DHS_KC;
-    const int64_t total = (int64_t)L * nob * nc * 1536;
-    const int64_t blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    hipLaunchKernelGGL(dhconv_pack_split_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc, adjoint);
+    if ((int64_t)nob * nc > 0x7fffffffLL || (L + 7) / 8 > 65535) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_pack_split_kernel, dim3((unsigned)(nob * nc), (unsigned)((L + 7) / 8)), dim3(256), 0, s, w,
+                       reinterpret_cast<unsigned int*>(packed), I, O, L, nob, nc, adjoint);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

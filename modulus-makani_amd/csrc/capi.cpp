@@ -445,7 +445,7 @@ extern "C" int sfno_dhconv(const sfno_dhconv_weights* w, const void* x, void* y,
     return sfno_spectral_to_coeffs(sout, y, (int64_t)batch * w->O, w->L, mmax, triangular, stream);
 }
 
-// ---- diagonal operator -----------------------------------------------------------------------------
+// ---- per-degree power (spectral losses) ----------------------------------------------------------------
 
 extern "C" int sfno_degree_power(const float* spec, float* power, int64_t rows, int lmax, int mmax, void* stream) {
     if (!spec || !power || !rows_ok(rows)) return SFNO_EINVAL;
@@ -456,6 +456,8 @@ extern "C" int sfno_degree_power_grad(const float* spec, const float* gpower, fl
     if (!spec || !gpower || !gspec || !rows_ok(rows)) return SFNO_EINVAL;
     return degree_power_grad_launch(spec, gpower, gspec, rows, lmax, mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream);
 }
+
+// ---- diagonal operator -----------------------------------------------------------------------------
 
 extern "C" int sfno_diagonal_contract(const void* x, const void* weight, void* y, int batch, int in_channels, int out_channels,
                                       int64_t positions, int adjoint, void* stream) {

@@ -1,7 +1,9 @@
-// dhconv on fp32 MFMA (v_mfma_f32_32x32x2_f32), gfx950.
+// dhconv on the matrix cores of gfx950:
 //
 //   y[b,o,l,m] = sum_i x[b,i,l,m] w[i,o,l]        (makani/models/common/contractions.py:130-136)
-// runs as real GEMMs per degree l on the spectral layout.  A complex product costs three real ones
+// as real GEMMs per degree l on the spectral layout.  Three kernels: dhconv_split_kernel (fp32 accuracy on the bf16
+// matrix pipe, the default, further down), dhconv_bf16_kernel (bf16 operands) and, first in this file, dhconv_kernel
+// on v_mfma_f32_32x32x2_f32, which serves odd channel counts.  In that one a complex product costs three real ones
 // (Gauss):  k1 = wr (xr + xi),  k2 = xr (wi - wr),  k3 = xi (wr + wi),  yr = k1 - k3,  yi = k1 + k2,
 // so each complex input channel feeds three MFMA operand pairs instead of the four of the 2x2 real
 // embedding, and a wavefront keeps three accumulators (K1, K2, K3) per tile that are combined when the

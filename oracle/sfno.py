@@ -47,6 +47,13 @@ class SfnoOracle:
             else:
                 residual = x
         y = self._conv(self.act(self._conv(x, sd, "encoder.fwd.0")), sd, "encoder.fwd.2")
+        # position embedding (sfnonet.py:612-622): a learnt field, or learnt coefficients synthesised on the input grid
+        if "pos_embed" in sd:
+            y = y + sd["pos_embed"].double()
+        elif "pos_embed.0" in sd:
+            re, im = sd["pos_embed.0"].double().numpy(), sd["pos_embed.1"].double().numpy()
+            c = re + 1j * np.pad(im, ((0, 0), (0, 0), (0, 0), (1, 0)))
+            y = y + torch.from_numpy(sht_inverse(c, self.up))
         for i in range(self.num_layers):
             fwd = self.down if i == 0 else self.mid
             inv = self.up if i == self.num_layers - 1 else self.mid
@@ -54,6 +61,8 @@ class SfnoOracle:
             w = sd[p + "filter.filter.weight"].numpy().astype(np.complex128)
             z, res = spectral_conv(y.numpy(), w, fwd, inv)
             z, res = torch.from_numpy(z), torch.from_numpy(np.asarray(res))
+            if p + "filter.filter.bias" in sd:           # spectral_convolution.py:143-144
+                z = z + sd[p + "filter.filter.bias"].double()
             z = self.act(self._norm(z, sd, p + "norm0"))
             if self.use_mlp:
                 z = self._conv(self.act(self._conv(z, sd, p + "mlp.fwd.0")), sd, p + "mlp.fwd.3")

@@ -51,6 +51,37 @@ def test_forward_matches_oracle_fp32(lib_built, case):
     assert rel_l2(y.cpu().double().numpy(), ref.numpy()) < 1e-4
 
 
+@pytest.mark.parametrize("extra", [dict(pos_embed="direct"), dict(pos_embed="frequency"), dict(bias="position"), dict(bias="constant")])
+def test_position_embedding_and_filter_bias(lib_built, extra):
+    """Learnt position embedding ("direct": a field on the input grid; "frequency": coefficients synthesised with the
+    up-sampling inverse transform, sfnonet.py:479-495, 612-622) and the SpectralConv bias (spectral_convolution.py:117-122,
+    143-144) against the oracle model, with the parameters set to random values (their defaults are zeros or tiny)."""
+    case = dict(inp_shape=(33, 64), out_shape=(33, 64), inp_chans=3, out_chans=2, scale_factor=2, embed_dim=16, num_layers=2)
+    print(f"case sfno {extra}", flush=True)
+    net = build(**case, **extra).cuda().eval()
+    g = torch.Generator().manual_seed(6)
+    with torch.no_grad():
+        for name, prm in net.named_parameters():
+            if "pos_embed" in name or name.endswith("filter.filter.bias"):
+                v = torch.randn(prm.shape, generator=g)
+                if name == "pos_embed.0":
+                    v = torch.tril(v, diagonal=0)
+                if name == "pos_embed.1":
+                    v = torch.tril(v, diagonal=-1)
+                prm.copy_(v)
+    x = torch.randn(2, 3, 33, 64, generator=g)
+    with torch.inference_mode():
+        y = net(x.cuda())
+    oracle = SfnoOracle(case["inp_shape"], case["out_shape"], 2, 2)
+    ref = oracle.forward(net.state_dict(), x)
+    assert rel_l2(y.cpu().double().numpy(), ref.numpy()) < 1e-4
+    # the extra parameters matter: without them the output differs (a bias that is constant over the grid does not:
+    # the instance norm that follows the filter removes it)
+    if extra != dict(bias="constant"):
+        sd0 = {k: v for k, v in net.state_dict().items() if "pos_embed" not in k and not k.endswith("filter.filter.bias")}
+        assert rel_l2(oracle.forward(sd0, x).numpy(), ref.numpy()) > 1e-2
+
+
 def test_forward_bf16_autocast(lib_built):
     """Under bf16 autocast only the pointwise layers run in bf16; the spectral path stays fp32.
 

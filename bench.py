@@ -35,7 +35,8 @@ def parse():
     ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--compute", default="fp32", choices=["fp32", "bf16", "fp32_mfma"],
-                    help="arithmetic of the Legendre and dhconv contractions: fp32 MFMA (reference precision) or bf16 MFMA inputs with fp32 accumulation")
+                    help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision; fp32 operands cut into three bf16 planes on the bf16 "
+                         "matrix pipe), fp32_mfma (transform pair only: the same on the fp32 matrix instruction) or bf16 MFMA inputs with fp32 accumulation")
     ap.add_argument("--rollout-steps", type=int, default=12, help="autoregressive steps timed by --workload rollout")
     ap.add_argument("--rollout-warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")

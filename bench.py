@@ -39,6 +39,7 @@ def parse():
                          "matrix pipe), fp32_mfma (transform pair only: the same on the fp32 matrix instruction) or bf16 MFMA inputs with fp32 accumulation")
     ap.add_argument("--rollout-steps", type=int, default=12, help="autoregressive steps timed by --workload rollout")
     ap.add_argument("--rollout-warmup", type=int, default=2)
+    ap.add_argument("--backward", action="store_true", help="--workload spectral_block: time forward + backward (input and weight gradients)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--yardstick", action="store_true",
                     help="also run one plain 256 MiB elementwise copy (mul by 1): the known-size reference for FETCH_SIZE/WRITE_SIZE runs")
@@ -256,6 +257,43 @@ def bench_spectral_block(args):
     with torch.no_grad():
         conv.weight.copy_(w.to(dev))
     x = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(2)).to(dev)
+    Tp = sum(min(l + 1, M) for l in range(L))
+    dh_flops = 8.0 * C * C * Tp
+    leg_flops = 4.0 * C * nlat * triangular_count(L, M)
+    if args.backward:
+        # forward + backward (input and weight gradients) through the adjoint kernels: twice the transform work and
+        # three times the channel mix of the forward pass
+        x.requires_grad_(True)
+        gy = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(6)).to(dev)
+
+        def step():
+            conv.weight.grad = None
+            x.grad = None
+            y, _ = conv(x)
+            y.backward(gy)
+            return y
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y = step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert torch.isfinite(x.grad).all() and torch.isfinite(torch.view_as_real(conv.weight.grad)).all()
+        flops = 3 * dh_flops + 4 * leg_flops
+        return {
+            "metric": "spectral block fwd+bwd/s @241x480x384",
+            "value": args.steps / dt,
+            "unit": "blocks/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32" if args.compute == "fp32" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic",
+            "config": {"workload": "configs[2] with its backward pass: SHT -> dhconv -> inverse SHT, gradients of the input and of the weight"},
+            "useful_TFLOPs_per_step": flops / 1e12,
+            "achieved_TFLOPs": flops / (dt / args.steps) / 1e12,
+        }
     with torch.no_grad():
         for _ in range(args.warmup):
             conv(x)
@@ -266,9 +304,6 @@ def bench_spectral_block(args):
         torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert torch.isfinite(y).all()
-    Tp = sum(min(l + 1, M) for l in range(L))
-    dh_flops = 8.0 * C * C * Tp
-    leg_flops = 4.0 * C * nlat * triangular_count(L, M)
     return {
         "metric": "spectral block fwd/s @241x480x384",
         "value": args.steps / dt,

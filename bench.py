@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SFNO spectral hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block|sfno8l|rollout|fft2_pair]
 
 Default workload (the configuration the headline metric is quoted on): forward + inverse
 real SHT at 721x1440 (equiangular, lmax = mmax = 721), batch 1, 73 channels, float32,
@@ -32,7 +32,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout"])
+    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--compute", default="fp32", choices=["fp32", "bf16", "fp32_mfma"],
                     help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision; fp32 operands cut into three bf16 planes on the bf16 "
@@ -241,6 +241,91 @@ def bench_sht_pair(args):
     return result
 
 
+def bench_fft2_pair(args):
+    """The planar pair RealFFT2 + InverseRealFFT2 (layers.py:219-287) at the full-resolution shape of configs[1], 720x1440."""
+    import torch
+    import makani_amd as ma
+    from makani_amd._lib import lib, check
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    nlat, nlon, C = 720, 1440, 73
+    fwd, inv = ma.RealFFT2(nlat, nlon), ma.InverseRealFFT2(nlat, nlon)
+    lmax, mmax = fwd.lmax, fwd.mmax
+    x = torch.randn(1, C, nlat, nlon, device=dev, generator=torch.Generator(dev).manual_seed(3))
+
+    def step():
+        return inv(fwd(x))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert float((y - x).abs().max()) < 1e-4
+
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    rows = C
+    pf, pi = fwd.plan(dev).handle, inv.plan(dev).handle
+    xm = torch.empty(lib.sfno_fourier_elems(pf, rows), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, rows), dtype=torch.float32, device=dev)
+    coeffs = torch.empty(1, C, lmax, mmax, dtype=torch.complex64, device=dev)
+    out = torch.empty_like(x)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    stages = {
+        "rfft": lambda: check(lib.sfno_rfft(pf, P(x), 0, P(xm), rows, sp), "rfft"),
+        "latitude_fft": lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), rows, sp), "latitude_fft"),
+        "spectral_to_coeffs": lambda: check(lib.sfno_spectral_to_coeffs(P(spec), P(coeffs), rows, lmax, mmax, 0, sp), "to_coeffs"),
+        "coeffs_to_spectral": lambda: check(lib.sfno_coeffs_to_spectral(P(coeffs), P(spec), rows, lmax, mmax, 0, sp), "to_spectral"),
+        "latitude_ifft": lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), rows, sp), "latitude_ifft"),
+        "irfft": lambda: check(lib.sfno_irfft(pi, P(xm), P(out), 0, rows, sp), "irfft"),
+    }
+    stage_ms = {name: event_time_ms(fn, max(5, args.steps), stream) for name, fn in stages.items()}
+    dom = max(("latitude_fft", "latitude_ifft"), key=lambda k: stage_ms[k])
+    lat_bytes = rows * mmax * (nlat + lmax) * 8          # every Fourier coefficient read once and every kept coefficient written once
+    gbs = lat_bytes / (stage_ms[dom] * 1e-3) / 1e9
+    result = {
+        "metric": "FFT2 fwd+inv/s @720x1440",
+        "value": args.steps / dt,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "RealFFT2 + InverseRealFFT2 (spectral_transform='fft'), 720x1440, all modes, batch 1, 73 channels, Gaussian random fields"},
+        "roofline": {"kernel": f"latfft_kernel ({dom})", "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": gbs / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes_per_launch": lat_bytes, "avg_launch_ms": stage_ms[dom]},
+        "stages_ms": stage_ms,
+    }
+    if not args.no_cpu_baseline:
+        from oracle.torch_ref import TorchRefFFT2
+
+        torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 1) <= 64 else 64)
+        ref = TorchRefFFT2(nlat, nlon)
+        xs = x[:, : 2 * args.cpu_sample_channels].cpu()
+        times = []
+        for it in range(4):
+            t0 = time.perf_counter()
+            ys = ref.inverse(ref.forward(xs))
+            if it:
+                times.append(time.perf_counter() - t0)
+        t = min(times)
+        n = xs.shape[1]
+        result["cpu_baseline"] = {"value": (1.0 / t) * (n / C), "unit": "pairs/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"{n} of {C} channels, torch.fft.rfft2 + irfft2 (the reference's own ops) in float32, best of 3 after "
+                                            f"1 warm-up ({t:.3f} s), scaled by {n}/{C}"}
+    return result
+
+
 def bench_spectral_block(args):
     """configs[2]: forward SHT -> dhconv -> inverse SHT on a 241x480 Legendre-Gauss grid, 384 channels."""
     import torch
@@ -424,6 +509,8 @@ def main():
             med, best, _, _ = time_sfno_forward(1, 10, 3, torch.device("cuda:0"))
             res["sfno_l8_fwd_ms_per_sample"] = {"value": med, "best": best, "batch": 1, "dtype": "bf16 pointwise / f32 spectral",
                                                 "config": "configs[3]: SFNO-linear 8 layers, embed 384, 721x1440, 73 channels, bf16 autocast"}
+    elif args.workload == "fft2_pair":
+        res = bench_fft2_pair(args)
     elif args.workload == "spectral_block":
         res = bench_spectral_block(args)
     elif args.workload == "sfno8l":

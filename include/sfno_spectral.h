@@ -48,6 +48,12 @@ extern "C" {
 #define SFNO_GRID_LEGENDRE_GAUSS 0
 #define SFNO_GRID_LOBATTO 1
 #define SFNO_GRID_EQUIANGULAR 2
+/* Not a quadrature rule: the planar pair RealFFT2 / InverseRealFFT2 of makani/models/common/layers.py:219-287
+ * (torch.fft.rfft2 / irfft2 with norm="ortho") behind the same plan and entry points.  The latitude stage is an
+ * FFT of length nlat; `lmax` <= nlat counts the kept latitude frequencies (the ceil(lmax/2) lowest non-negative
+ * and the floor(lmax/2) highest, in that order, as the reference concatenates them), `mmax` <= nlon/2+1 the
+ * kept longitude frequencies.  `norm` and `csphase` are ignored, the spectral layout is full (no l < m rule). */
+#define SFNO_GRID_PLANAR 3
 
 /* norm = normalisation of the harmonics (torch-harmonics `norm=` strings) */
 #define SFNO_NORM_ORTHO 0

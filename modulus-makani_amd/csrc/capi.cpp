@@ -1,4 +1,5 @@
 // C ABI of libsfno_spectral: plan management and the enqueue-only compute entry points.
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <new>
@@ -95,6 +96,42 @@ PgemmArgs legendre_args(const sfno_sht_plan* p, const PgemmTable& t, const float
 
 bool rows_ok(int64_t rows) { return rows > 0 && sfno_spectral_ld(rows) < (int64_t)1 << 30; }
 
+// Planar plans (SFNO_GRID_PLANAR).  The longitude kernels are those of the spherical transforms,
+//   F: x -> s * sum_n x_n e^{-i m phi_n} (s = 2 pi / nlon)   and   C: the unnormalised complex-to-real transform,
+// so torch.fft.rfft2(norm="ortho") is  a * (latitude DFT) o F  with a = 1 / (s sqrt(nlat nlon)), and
+// torch.fft.irfft2(norm="ortho") is  C o b * (inverse latitude DFT)  with b = 1 / sqrt(nlat nlon).  The unnormalised
+// latitude DFT pair are each other's conjugate transposes; with F^T = s C o diag(1, 1/2, ..., 1/2, 1) and
+// C^T = diag(1, 2, ..., 2, 1) o F / s the adjoint of either transform is the other one with order weights.
+enum { MS_FWD = 0, MS_INV = 1, MS_FWD_ADJ = 2, MS_INV_ADJ = 3 };
+
+int planar_init(sfno_sht_plan* p) {
+    int rc = fft_plan_init(p->fft, p->nlon);
+    if (rc == SFNO_OK) rc = fft_plan_init(p->fft_lat, p->nlat);
+    if (rc != SFNO_OK) return rc;
+    const double s = 2.0 * 3.14159265358979323846264338327950288 / p->nlon;
+    const double b = 1.0 / std::sqrt((double)p->nlat * (double)p->nlon), a = b / s;
+    const bool even = p->nlon % 2 == 0;
+    const int bits[4] = {SFNO_DIR_FORWARD, SFNO_DIR_INVERSE, SFNO_DIR_FORWARD_ADJOINT, SFNO_DIR_INVERSE_ADJOINT};
+    for (int d = 0; d < 4; ++d) {
+        if (!(p->directions & bits[d])) continue;
+        std::vector<float> ms(p->mmax);
+        for (int m = 0; m < p->mmax; ++m) {
+            const bool edge = m == 0 || (even && m == p->nlon / 2);
+            ms[m] = (float)(d == MS_FWD ? a : d == MS_INV ? b : d == MS_FWD_ADJ ? b * (edge ? 1.0 : 0.5) : a * (edge ? 1.0 : 2.0));
+        }
+        if ((rc = upload(&p->d_mscale[d], ms)) != SFNO_OK) return rc;
+    }
+    return SFNO_OK;
+}
+
+// latitude stage of a planar plan: `which` selects the order factors, `inverse` the direction of the latitude FFT
+int planar_stage(const sfno_sht_plan* p, int which, bool inverse, const float* in, float* out, int64_t rows, void* stream) {
+    if (!p->d_mscale[which]) return SFNO_EINVAL;
+    return latfft_launch(p->fft_lat, inverse, in, out, p->mmax, p->lmax, (int)sfno_spectral_ld(rows), p->d_mscale[which], (hipStream_t)stream);
+}
+
+bool planar(const sfno_sht_plan* p) { return p->grid == SFNO_GRID_PLANAR; }
+
 }  // namespace
 
 extern "C" const char* sfno_strerror(int code) {
@@ -130,7 +167,8 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if ((directions & (SFNO_DIR_FORWARD | SFNO_DIR_FORWARD_ADJOINT)) && mmax > nlon / 2 + 1) return SFNO_EINVAL;
     // the adjoint of the zero-padding inverse would need Fourier bins the real FFT does not produce
     if ((directions & SFNO_DIR_INVERSE_ADJOINT) && mmax > nlon / 2 + 1) return SFNO_EUNSUPPORTED;
-    if (grid < 0 || grid > 2 || norm < 0 || norm > 2) return SFNO_EINVAL;
+    if (grid < 0 || grid > SFNO_GRID_PLANAR || norm < 0 || norm > 2) return SFNO_EINVAL;
+    if (grid == SFNO_GRID_PLANAR && (lmax > nlat || mmax > nlon / 2 + 1)) return SFNO_EINVAL;
     if (!(directions & all_dirs) || (directions & ~all_dirs)) return SFNO_EINVAL;
     if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16 && compute != SFNO_COMPUTE_FP32_MFMA) return SFNO_EUNSUPPORTED;
     sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
@@ -141,6 +179,12 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     p->compute = compute == SFNO_COMPUTE_BF16 ? SFNO_COMPUTE_BF16 : SFNO_COMPUTE_FP32;
     p->format = compute == SFNO_COMPUTE_BF16 ? PG_FORMAT_BF16 : compute == SFNO_COMPUTE_FP32_MFMA ? PG_FORMAT_FP32 : PG_FORMAT_SPLIT;
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return SFNO_EHIP; }
+    if (grid == SFNO_GRID_PLANAR) {
+        int rc = planar_init(p);
+        if (rc != SFNO_OK) { sfno_sht_plan_destroy(p); return rc; }
+        *out = p;
+        return SFNO_OK;
+    }
     std::vector<double> theta(nlat), w(nlat);
     int rc = quadrature(grid, nlat, theta.data(), w.data());
     if (rc == SFNO_OK) rc = fft_plan_init(p->fft, nlon);
@@ -176,6 +220,9 @@ extern "C" int sfno_sht_plan_destroy(sfno_sht_plan* p) {
     free_table(p->fwd_adj);
     free_table(p->inv_adj);
     fft_plan_free(p->fft);
+    fft_plan_free(p->fft_lat);
+    for (float*& d : p->d_mscale)
+        if (d) { (void)hipFree(d); d = nullptr; }
     delete p;
     return SFNO_OK;
 }
@@ -209,6 +256,7 @@ extern "C" int sfno_irfft(const sfno_sht_plan* p, const float* xm, void* x, int 
 extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, float* spec, int64_t rows, void* stream) {
     if (!p || !xm || !spec || !rows_ok(rows)) return SFNO_EINVAL;
     if (!(p->directions & SFNO_DIR_FORWARD)) return SFNO_EINVAL;
+    if (planar(p)) return planar_stage(p, MS_FWD, false, xm, spec, rows, stream);
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->fwd, xm, spec, ld);
     return legendre_fold_launch(true, p->format, a, p->fwd.n_work, (hipStream_t)stream);
@@ -217,6 +265,7 @@ extern "C" int sfno_legendre_analysis(const sfno_sht_plan* p, const float* xm, f
 extern "C" int sfno_legendre_synthesis(const sfno_sht_plan* p, const float* spec, float* xm, int64_t rows, void* stream) {
     if (!p || !xm || !spec || !rows_ok(rows)) return SFNO_EINVAL;
     if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
+    if (planar(p)) return planar_stage(p, MS_INV, true, spec, xm, rows, stream);
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv, spec, xm, ld);
     return legendre_fold_launch(false, p->format, a, p->inv.n_work, (hipStream_t)stream);
@@ -252,7 +301,7 @@ extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* co
     int rc = sfno_sht_analysis(p, x, SFNO_DTYPE_F32, w.spec, rows, workspace, workspace_bytes, stream);
     if (rc != SFNO_OK) return rc;
     return spectral_to_coeffs_launch(w.spec, reinterpret_cast<float2*>(coeffs), rows, p->lmax, p->mmax,
-                                     (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+                                     (int)sfno_spectral_ld(rows), planar(p) ? 0 : 1, (hipStream_t)stream);
 }
 
 extern "C" int sfno_sht_inverse(const sfno_sht_plan* p, const void* coeffs, float* x, int64_t rows, void* workspace,
@@ -261,7 +310,7 @@ extern "C" int sfno_sht_inverse(const sfno_sht_plan* p, const void* coeffs, floa
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     int rc = coeffs_to_spectral_launch(reinterpret_cast<const float2*>(coeffs), w.spec, rows, p->lmax, p->mmax,
-                                       (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+                                       (int)sfno_spectral_ld(rows), planar(p) ? 0 : 1, (hipStream_t)stream);
     if (rc != SFNO_OK) return rc;
     return sfno_sht_synthesis(p, w.spec, x, SFNO_DTYPE_F32, rows, workspace, workspace_bytes, stream);
 }
@@ -275,8 +324,13 @@ extern "C" int sfno_sht_analysis_adjoint(const sfno_sht_plan* p, const float* gs
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     const int64_t ld = sfno_spectral_ld(rows);
-    PgemmArgs a = legendre_args(p, p->fwd_adj, gspec, w.xm, ld);
-    int rc = legendre_fold_launch(false, p->format, a, p->fwd_adj.n_work, (hipStream_t)stream);
+    int rc;
+    if (planar(p)) {
+        rc = planar_stage(p, MS_FWD_ADJ, true, gspec, w.xm, rows, stream);
+    } else {
+        PgemmArgs a = legendre_args(p, p->fwd_adj, gspec, w.xm, ld);
+        rc = legendre_fold_launch(false, p->format, a, p->fwd_adj.n_work, (hipStream_t)stream);
+    }
     if (rc != SFNO_OK) return rc;
     return sfno_irfft(p, w.xm, gx, x_dtype, rows, stream);
 }
@@ -289,6 +343,7 @@ extern "C" int sfno_sht_synthesis_adjoint(const sfno_sht_plan* p, const void* gx
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     int rc = sfno_rfft(p, gx, x_dtype, w.xm, rows, stream);
     if (rc != SFNO_OK) return rc;
+    if (planar(p)) return planar_stage(p, MS_INV_ADJ, false, w.xm, gspec, rows, stream);
     const int64_t ld = sfno_spectral_ld(rows);
     PgemmArgs a = legendre_args(p, p->inv_adj, w.xm, gspec, ld);
     return legendre_fold_launch(true, p->format, a, p->inv_adj.n_work, (hipStream_t)stream);
@@ -300,7 +355,7 @@ extern "C" int sfno_sht_forward_adjoint(const sfno_sht_plan* p, const void* gcoe
     Ws w = carve(p, rows, workspace);
     if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
     int rc = coeffs_to_spectral_launch(reinterpret_cast<const float2*>(gcoeffs), w.spec, rows, p->lmax, p->mmax,
-                                       (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+                                       (int)sfno_spectral_ld(rows), planar(p) ? 0 : 1, (hipStream_t)stream);
     if (rc != SFNO_OK) return rc;
     return sfno_sht_analysis_adjoint(p, w.spec, gx, SFNO_DTYPE_F32, rows, workspace, workspace_bytes, stream);
 }
@@ -313,7 +368,7 @@ extern "C" int sfno_sht_inverse_adjoint(const sfno_sht_plan* p, const float* gx,
     int rc = sfno_sht_synthesis_adjoint(p, gx, SFNO_DTYPE_F32, w.spec, rows, workspace, workspace_bytes, stream);
     if (rc != SFNO_OK) return rc;
     return spectral_to_coeffs_launch(w.spec, reinterpret_cast<float2*>(gcoeffs), rows, p->lmax, p->mmax,
-                                     (int)sfno_spectral_ld(rows), 1, (hipStream_t)stream);
+                                     (int)sfno_spectral_ld(rows), planar(p) ? 0 : 1, (hipStream_t)stream);
 }
 
 extern "C" int sfno_coeffs_to_spectral(const void* coeffs, float* spec, int64_t rows, int lmax, int mmax, int triangular,

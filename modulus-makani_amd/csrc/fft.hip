@@ -36,25 +36,30 @@ __device__ __forceinline__ float2 twid(const float2* __restrict__ tw, int idx) {
 // One Stockham pass of radix R over `nseq` sequences of length n held in LDS.
 // For butterfly j (0 <= j < n/R), with ns = product of the radices already applied and
 // k = j mod ns:  v[r] = in[j + r n/R] * w^(r k n/(ns R)),  out[(j-k) R + k + q ns] = DFT_R(v)[q].
-template <int R, int INV>
+// COL = false: sequence sq occupies [sq n, sq n + n) (longitude transforms: a sequence is a grid row);
+// COL = true: element i of sequence sq sits at i nseq + sq (latitude transforms: the sequences are the
+// channels of one order, contiguous in HBM and in LDS).  Either way neighbouring lanes touch neighbouring words.
+template <int R, int INV, bool COL>
 __device__ __forceinline__ void pass_fixed(const float2* __restrict__ in, float2* __restrict__ out, const float2* __restrict__ tw,
                                            int n, int ns, int nseq, int tid, int nthreads) {
     const int nb = n / R;
     const int tstep = n / (ns * R);
+    const int es = COL ? nseq : 1;                    // distance between consecutive elements of a sequence
     for (int e = tid; e < nseq * nb; e += nthreads) {
-        const int sq = e / nb, j = e - sq * nb;
+        const int sq = COL ? e % nseq : e / nb, j = COL ? e / nseq : e - sq * nb;
         const int k = j % ns;
-        const float2* src = in + sq * n + j;
+        const float2* src = in + (COL ? sq : sq * n) + j * es;
         float2 v[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            v[r] = src[r * nb];
+            v[r] = src[r * nb * es];
             if (r > 0) v[r] = cmul(v[r], twid<INV>(tw, (r * k * tstep) % n));
         }
-        float2* dst = out + sq * n + (j - k) * R + k;
+        float2* dst = out + (COL ? sq : sq * n) + ((j - k) * R + k) * es;
+        const int os = ns * es;                        // distance between the outputs of the butterfly
         if (R == 2) {
             dst[0] = cadd(v[0], v[1]);
-            dst[ns] = csub(v[0], v[1]);
+            dst[os] = csub(v[0], v[1]);
         } else if (R == 3) {
             const float s3 = 0.86602540378443864676f;
             float2 t1 = cadd(v[1], v[2]);
@@ -62,15 +67,15 @@ __device__ __forceinline__ void pass_fixed(const float2* __restrict__ in, float2
             float2 d = csub(v[1], v[2]);
             float2 t3 = mul_mi<INV>(make_float2(s3 * d.x, s3 * d.y));
             dst[0] = cadd(v[0], t1);
-            dst[ns] = cadd(t2, t3);
-            dst[2 * ns] = csub(t2, t3);
+            dst[os] = cadd(t2, t3);
+            dst[2 * os] = csub(t2, t3);
         } else if (R == 4) {
             float2 a0 = cadd(v[0], v[2]), a1 = csub(v[0], v[2]);
             float2 a2 = cadd(v[1], v[3]), a3 = mul_mi<INV>(csub(v[1], v[3]));
             dst[0] = cadd(a0, a2);
-            dst[ns] = cadd(a1, a3);
-            dst[2 * ns] = csub(a0, a2);
-            dst[3 * ns] = csub(a1, a3);
+            dst[os] = cadd(a1, a3);
+            dst[2 * os] = csub(a0, a2);
+            dst[3 * os] = csub(a1, a3);
         } else if (R == 5) {
             const float c1 = 0.30901699437494742410f, c2 = -0.80901699437494742410f;
             const float s1 = 0.95105651629515357212f, s2 = 0.58778525229247312917f;
@@ -81,34 +86,44 @@ __device__ __forceinline__ void pass_fixed(const float2* __restrict__ in, float2
             float2 f1 = mul_mi<INV>(make_float2(s1 * m1.x + s2 * m2.x, s1 * m1.y + s2 * m2.y));
             float2 f2 = mul_mi<INV>(make_float2(s2 * m1.x - s1 * m2.x, s2 * m1.y - s1 * m2.y));
             dst[0] = cadd(v[0], cadd(p1, p2));
-            dst[ns] = cadd(e1, f1);
-            dst[2 * ns] = cadd(e2, f2);
-            dst[3 * ns] = csub(e2, f2);
-            dst[4 * ns] = csub(e1, f1);
+            dst[os] = cadd(e1, f1);
+            dst[2 * os] = cadd(e2, f2);
+            dst[3 * os] = csub(e2, f2);
+            dst[4 * os] = csub(e1, f1);
         }
     }
 }
 
 // Any other (prime) radix: direct O(R^2) butterfly straight from LDS, no private arrays.
-template <int INV>
+template <int INV, bool COL>
 __device__ __forceinline__ void pass_generic(const float2* __restrict__ in, float2* __restrict__ out, const float2* __restrict__ tw,
                                              int n, int ns, int R, int nseq, int tid, int nthreads) {
     const int nb = n / R;
     const int tstep = n / (ns * R);
     const int rstep = n / R;
+    const int es = COL ? nseq : 1;
     for (int e = tid; e < nseq * nb * R; e += nthreads) {
-        const int q = e % R;
-        const int e2 = e / R;
-        const int sq = e2 / nb, j = e2 - sq * nb;
+        int q, sq, j;
+        if (COL) {
+            sq = e % nseq;
+            const int e2 = e / nseq;
+            q = e2 % R;
+            j = e2 / R;
+        } else {
+            q = e % R;
+            const int e2 = e / R;
+            sq = e2 / nb;
+            j = e2 - sq * nb;
+        }
         const int k = j % ns;
-        const float2* src = in + sq * n + j;
+        const float2* src = in + (COL ? sq : sq * n) + j * es;
         float2 acc = make_float2(0.f, 0.f);
         for (int r = 0; r < R; ++r) {
             // input twiddle w^(r k tstep) and butterfly factor w^(r q n/R)
             int idx = (int)(((long long)r * k * tstep + (long long)((r * q) % R) * rstep) % n);
-            acc = cadd(acc, cmul(src[r * nb], twid<INV>(tw, idx)));
+            acc = cadd(acc, cmul(src[r * nb * es], twid<INV>(tw, idx)));
         }
-        out[sq * n + (j - k) * R + k + q * ns] = acc;
+        out[(COL ? sq : sq * n) + ((j - k) * R + k + q * ns) * es] = acc;
     }
 }
 
@@ -118,7 +133,7 @@ struct FftDev {
     int radix[24];
 };
 
-template <int INV>
+template <int INV, bool COL = false>
 __device__ __forceinline__ float2* run_passes(const FftDev& f, float2* buf0, float2* buf1, int nseq, int tid, int nthreads) {
     int ns = 1;
     float2* in = buf0;
@@ -126,11 +141,11 @@ __device__ __forceinline__ float2* run_passes(const FftDev& f, float2* buf0, flo
     for (int p = 0; p < f.npass; ++p) {
         const int R = f.radix[p];
         switch (R) {
-            case 2: pass_fixed<2, INV>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
-            case 3: pass_fixed<3, INV>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
-            case 4: pass_fixed<4, INV>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
-            case 5: pass_fixed<5, INV>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
-            default: pass_generic<INV>(in, out, f.tw, f.n, ns, R, nseq, tid, nthreads); break;
+            case 2: pass_fixed<2, INV, COL>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
+            case 3: pass_fixed<3, INV, COL>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
+            case 4: pass_fixed<4, INV, COL>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
+            case 5: pass_fixed<5, INV, COL>(in, out, f.tw, f.n, ns, nseq, tid, nthreads); break;
+            default: pass_generic<INV, COL>(in, out, f.tw, f.n, ns, R, nseq, tid, nthreads); break;
         }
         ns *= R;
         __syncthreads();
@@ -261,6 +276,74 @@ static FftDev make_dev(const FftPlan& p) {
 
 // LDS budget per workgroup (bytes) the FFT kernels may ask for
 static const size_t kFftMaxLds = 160 * 1024;
+
+// Latitude FFT of the planar transform pair (RealFFT2 / InverseRealFFT2, makani/models/common/layers.py:219-287):
+// the second dimension of torch.fft.rfft2 / irfft2 with the reference's mode truncation.  Both sides use the
+// order-major layout: in[m][k][ld] -> out[m][j][ld], channels contiguous.  A workgroup transforms 2^cshift complex
+// channels of one order; the sequences stay channel-contiguous in LDS.
+//   INV = 0: k = latitude (n rows), j = kept frequency (lmax rows): j < ceil(lmax/2) is frequency j, the rest are
+//            the floor(lmax/2) highest (negative) frequencies n - lmax + j.
+//   INV = 1: k = kept frequency, j = latitude; dropped frequencies are zero.
+// Every output is multiplied by mscale[m] (normalisation, and the order weights of the adjoint transforms).
+// grid = (mmax, ceil(ld / 2 / 2^cshift)); dynamic LDS = 2 * n * 2^cshift * sizeof(float2)
+constexpr int LATFFT_THREADS = 512;
+
+template <int INV>
+__global__ __launch_bounds__(LATFFT_THREADS) void latfft_kernel(FftDev f, const float* __restrict__ in, float* __restrict__ out, int lmax, int ld,
+                                                                int cshift, const float* __restrict__ mscale) {
+    extern __shared__ __align__(16) float2 lds[];
+    const int n = f.n, tid = threadIdx.x, cw = 1 << cshift;
+    const int m = blockIdx.x, c0 = blockIdx.y * cw;
+    const int lhigh = (lmax + 1) / 2, gap = n - lmax;
+    float2* buf0 = lds;
+    float2* buf1 = lds + n * cw;
+    const int nin = INV ? lmax : n, nout = INV ? n : lmax;
+    for (int e = tid; e < n * cw; e += LATFFT_THREADS) {
+        const int i = e >> cshift, c = e & (cw - 1);
+        // row of the input that lands on element i of the sequence (-1: a dropped frequency)
+        const int k = !INV ? i : i < lhigh ? i : i >= lhigh + gap ? i - gap : -1;
+        float2 v = make_float2(0.f, 0.f);
+        if (k >= 0 && 2 * (c0 + c) < ld) v = *reinterpret_cast<const float2*>(in + ((int64_t)m * nin + k) * ld + 2 * (c0 + c));
+        buf0[e] = v;
+    }
+    __syncthreads();
+    const float2* z = run_passes<INV, true>(f, buf0, buf1, cw, tid, LATFFT_THREADS);
+    const float sc = mscale[m];
+    for (int e = tid; e < nout * cw; e += LATFFT_THREADS) {
+        const int j = e >> cshift, c = e & (cw - 1);
+        const int i = INV ? j : j < lhigh ? j : j + gap;
+        if (2 * (c0 + c) >= ld) continue;
+        const float2 v = z[i * cw + c];
+        *reinterpret_cast<float2*>(out + ((int64_t)m * nout + j) * ld + 2 * (c0 + c)) = make_float2(sc * v.x, sc * v.y);
+    }
+}
+
+int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
+    if (lmax < 1 || lmax > p.n || mmax < 1 || ld % 2 != 0 || !mscale) return SFNO_EINVAL;
+    if (fft_fast_supported(p.n)) {
+        const int rc = latfft_fast_launch(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        if (rc != SFNO_EUNSUPPORTED) return rc;
+    }
+    // as many channels per workgroup as the two LDS buffers allow, at most 8 (one 64-byte line per row)
+    int cshift = 3;
+    while (cshift > 0 && (2 * sizeof(float2) * p.n << cshift) > kFftMaxLds) --cshift;
+    const size_t lds = 2 * sizeof(float2) * p.n << cshift;
+    if (lds > kFftMaxLds) return SFNO_EUNSUPPORTED;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)latfft_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess ||
+            hipFuncSetAttribute((const void*)latfft_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess)
+            return SFNO_EHIP;
+        attr_set = true;
+    }
+    const int cw = 1 << cshift;
+    dim3 grid(mmax, (unsigned)((ld / 2 + cw - 1) / cw));
+    if (inverse)
+        hipLaunchKernelGGL(latfft_kernel<1>, grid, dim3(LATFFT_THREADS), lds, s, make_dev(p), in, out, lmax, ld, cshift, mscale);
+    else
+        hipLaunchKernelGGL(latfft_kernel<0>, grid, dim3(LATFFT_THREADS), lds, s, make_dev(p), in, out, lmax, ld, cshift, mscale);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
 
 template <int PAIRS>
 static int rfft_go(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {

@@ -1,5 +1,6 @@
-// Specialised longitude FFTs for the transform lengths the SFNO uses (1440 = 16*10*9,
-// 480 = 10*16*3, ...): everything about the length is a compile-time constant.
+// Specialised FFTs for the transform lengths the SFNO uses (1440 = 16*10*9, 480 = 10*16*3, ...),
+// along longitude and, for the planar transform pair, along latitude: everything about the
+// length is a compile-time constant.
 //
 // A workgroup transforms S complex sequences (2*S channels at one latitude) held in LDS.
 // The length factors as N = R0*R1*R2 and every pass is one radix-R butterfly per thread,
@@ -447,11 +448,65 @@ __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict
     }
 }
 
+// ---- latitude FFT of the planar transform pair -------------------------------------------------------------
+// in[m][k][ld] -> out[m][j][ld] on the order-major layout (see latfft_launch): a workgroup transforms the LS = 8
+// complex channels of one 64-byte line of every row of one order.  Rows arrive channel-contiguous and are
+// transposed on the way into LDS, where each channel is one sequence of the in-place passes above.
+//   INV = 0: decimation in frequency; kept frequency f leaves from slot pos(f).
+//   INV = 1: decimation in time; kept frequency f enters at slot pos(f), dropped frequencies enter as zeros.
+// grid = (mmax, ceil(ld / 16))
+constexpr int LS = 8;
+
+template <int N, int R0, int R1, int R2, int FT, int INV>
+__global__ __launch_bounds__(FT) void latfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ in,
+                                                         float* __restrict__ out, int lmax, int ld, const float* __restrict__ mscale) {
+    using G = Geo<N, R0, R1, R2>;
+    __shared__ __align__(16) float2 z[LS * G::PITCH];
+    const int tid = threadIdx.x;
+    const int m = blockIdx.x, c0 = blockIdx.y * LS;
+    const int lhigh = (lmax + 1) / 2, gap = N - lmax;
+    const int nin = INV ? lmax : N, nout = INV ? N : lmax;
+    const int c = tid & (LS - 1);
+    const bool live = 2 * (c0 + c) < ld;
+    const float* src = in + (int64_t)m * nin * ld + 2 * (c0 + c);
+    {
+        // all global loads of the workgroup are issued before the first LDS store
+        constexpr int TOT = LS * N, IT = (TOT + FT - 1) / FT;
+        float2 v[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int i = (tid + it * FT) / LS;
+            // row of the input that belongs to element i of the sequence (-1: a dropped frequency)
+            const int k = !INV ? i : i < lhigh ? i : i >= lhigh + gap ? i - gap : -1;
+            v[it] = make_float2(0.f, 0.f);
+            if (i < N && k >= 0 && live) v[it] = *reinterpret_cast<const float2*>(src + (int64_t)k * ld);
+        }
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int i = (tid + it * FT) / LS;
+            if (i < N) z[c * G::PITCH + (INV ? G::pos(i) : i)] = v[it];
+        }
+    }
+    __syncthreads();
+    if (INV)
+        passes_dit<N, R0, R1, R2, LS, FT>(z, tw0, tw1, tid);
+    else
+        passes_dif<N, R0, R1, R2, LS, FT>(z, tw0, tw1, tid);
+    if (!live) return;
+    const float sc = mscale[m];
+    float* dst = out + (int64_t)m * nout * ld + 2 * (c0 + c);
+    for (int j = tid / LS; j < nout; j += FT / LS) {
+        const int i = INV ? j : G::pos(j < lhigh ? j : j + gap);
+        const float2 v = z[c * G::PITCH + i];
+        *reinterpret_cast<float2*>(dst + (int64_t)j * ld) = make_float2(sc * v.x, sc * v.y);
+    }
+}
+
 struct FastEntry {
     int n, r0, r1, r2;
 };
 // lengths with a specialised kernel; the last radix acts on contiguous groups, an odd one keeps LDS banks apart
-const FastEntry kFast[] = {{1440, 16, 10, 9}, {480, 10, 16, 3}, {64, 8, 8, 1}, {180, 4, 5, 9}};
+const FastEntry kFast[] = {{1440, 16, 10, 9}, {720, 16, 5, 9}, {480, 10, 16, 3}, {240, 16, 5, 3}, {64, 8, 8, 1}, {180, 4, 5, 9}};
 
 const FastEntry* find_fast(int n) {
     for (const auto& e : kFast)
@@ -478,9 +533,31 @@ int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t r
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
+template <int N, int R0, int R1, int R2>
+int go_lat(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
+    constexpr int FT = (LS * N >= 4096) ? 512 : 256;
+    dim3 grid(mmax, (unsigned)((ld / 2 + LS - 1) / LS));
+    if (inverse)
+        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 1>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, lmax, ld, mscale);
+    else
+        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 0>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, lmax, ld, mscale);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
 }  // namespace
 
 bool fft_fast_supported(int n) { return find_fast(n) != nullptr; }
+
+int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
+    switch (p.n) {
+        case 720: return go_lat<720, 16, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 480: return go_lat<480, 10, 16, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 240: return go_lat<240, 16, 5, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 180: return go_lat<180, 4, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 64: return go_lat<64, 8, 8, 1>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+    }
+    return SFNO_EUNSUPPORTED;
+}
 
 int fft_fast_plan_init(FftPlan& p) {
     const FastEntry* f = find_fast(p.n);
@@ -515,7 +592,9 @@ int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, i
                   : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, s);
     switch (p.n) {
         FF_CASE(1440, 16, 10, 9)
+        FF_CASE(720, 16, 5, 9)
         FF_CASE(480, 10, 16, 3)
+        FF_CASE(240, 16, 5, 3)
         FF_CASE(64, 8, 8, 1)
         FF_CASE(180, 4, 5, 9)
     }

@@ -134,12 +134,17 @@ int fft_fast_plan_init(FftPlan& p);
 // grid_dtype: element type of the grid-side tensor (SFNO_DTYPE_*); the Fourier side is always float
 int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
                     hipStream_t s);
+// latitude FFT on the specialised passes; SFNO_EUNSUPPORTED for a length without them
+int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s);
 int fft_plan_init(FftPlan& p, int n);
 void fft_plan_free(FftPlan& p);
 // x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon
 int rfft_launch(const FftPlan& p, const void* x, int x_dtype, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
 // xm [mmax][nlat][ld] -> x [rows][nlat][nlon]
 int irfft_launch(const FftPlan& p, const float* xm, void* x, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+// latitude FFT of the planar transforms on the order-major layout: in[m][nlat | lmax][ld] -> out[m][lmax | nlat][ld]
+// (forward keeps lmax frequencies, inverse zero-fills the dropped ones); outputs are multiplied by mscale[m] (device array)
+int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s);
 
 // ---- per-degree power of spectral-layout coefficients and its gradient (degree_power.hip) ------------
 int degree_power_launch(const float* spec, float* power, int64_t rows, int lmax, int mmax, int ld, hipStream_t s);
@@ -160,6 +165,9 @@ struct sfno_sht_plan {
     sfno::PgemmTable fwd, inv;          // analysis (forward) and synthesis (inverse) streams
     sfno::PgemmTable fwd_adj, inv_adj;  // their adjoints: synthesis-format stream of the analysis table and vice versa
     sfno::FftPlan fft;
+    // grid == SFNO_GRID_PLANAR: the latitude stage is an FFT of length nlat instead of a Legendre stream
+    sfno::FftPlan fft_lat;
+    float* d_mscale[4] = {nullptr, nullptr, nullptr, nullptr};   // per-order output factors: forward, inverse, forward adjoint, inverse adjoint
 };
 
 struct sfno_dhconv_weights {

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsfno_spectral.so")
 
-GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2}
+GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2, "planar": 3}
 NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
 DIR_FORWARD, DIR_INVERSE, DIR_FORWARD_ADJOINT, DIR_INVERSE_ADJOINT = 1, 2, 4, 8
 COMPUTE_FP32, COMPUTE_BF16, COMPUTE_FP32_MFMA = 0, 1, 2

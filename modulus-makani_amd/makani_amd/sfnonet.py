@@ -17,6 +17,7 @@ import torch.nn as nn
 
 from . import pointwise as pw
 from .sht import RealSHT, InverseRealSHT
+from .layers import RealFFT2, InverseRealFFT2
 from .spectral_convolution import SpectralConv
 
 _ACTIVATIONS = {"relu": nn.ReLU, "gelu": nn.GELU, "silu": nn.SiLU}
@@ -230,8 +231,9 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         super().__init__()
         # spectral_compute = "bf16" (not a Makani option) runs the Legendre and dhconv contractions on bf16 MFMA
         self.spectral_compute = spectral_compute
-        if spectral_transform != "sht":
-            raise NotImplementedError("only spectral_transform='sht' runs on the HIP path")
+        if spectral_transform not in ("sht", "fft"):
+            raise ValueError("Unknown spectral transform")
+        self.spectral_transform = spectral_transform
         self.inp_shape, self.out_shape = tuple(inp_shape), tuple(out_shape)
         self.inp_chans, self.out_chans, self.embed_dim = inp_chans, out_chans, embed_dim
         self.repeat_layers, self.big_skip = repeat_layers, big_skip
@@ -296,6 +298,16 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
             modes_lat = int(self.h * hard_thresholding_fraction)
             modes_lon = int((self.w // 2 + 1) * hard_thresholding_fraction)
         c = self.spectral_compute
+        if self.spectral_transform == "fft":
+            # planar pair (sfnonet.py:542-556); the grid type arguments do not apply
+            self.trans_down = RealFFT2(*self.inp_shape, lmax=modes_lat, mmax=modes_lon).float()
+            self.itrans_up = InverseRealFFT2(*self.out_shape, lmax=modes_lat, mmax=modes_lon).float()
+            self.trans = RealFFT2(self.h, self.w, lmax=modes_lat, mmax=modes_lon).float()
+            self.itrans = InverseRealFFT2(self.h, self.w, lmax=modes_lat, mmax=modes_lon).float()
+            self.inp_shape_loc = (self.trans_down.nlat, self.trans_down.nlon)
+            self.out_shape_loc = (self.itrans_up.nlat, self.itrans_up.nlon)
+            self.h_loc, self.w_loc = self.itrans.nlat, self.itrans.nlon
+            return
         self.trans_down = RealSHT(*self.inp_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type, compute=c).float()
         self.itrans_up = InverseRealSHT(*self.out_shape, lmax=modes_lat, mmax=modes_lon, grid=model_grid_type, compute=c).float()
         self.trans = RealSHT(self.h, self.w, lmax=modes_lat, mmax=modes_lon, grid=sht_grid_type, compute=c).float()

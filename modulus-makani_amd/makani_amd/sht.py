@@ -92,6 +92,7 @@ def _ptr(t):
 class _SHTBase(nn.Module):
     _directions = 0
     _adjoint_direction = 0
+    _planar = False    # True in the planar FFT pair of layers.py, which shares the plan, layouts and entry points
 
     def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, compute="fp32"):
         super().__init__()
@@ -111,6 +112,8 @@ class _SHTBase(nn.Module):
             self.lmax = lmax or self.nlat
         elif grid == "lobatto":
             self.lmax = lmax or self.nlat - 1
+        elif grid == "planar" and self._planar:
+            self.lmax = lmax or self.nlat
         else:
             raise ValueError("Unknown quadrature mode")
         if norm not in _lib.NORM:

@@ -68,7 +68,10 @@ class SpectralConv(nn.Module):
             and isinstance(inverse_transform, InverseRealSHT)
             and forward_transform.lmax == inverse_transform.lmax
             and forward_transform.mmax == inverse_transform.mmax
+            and forward_transform._planar == inverse_transform._planar
         )
+        # coefficients of a spherical transform vanish for l < m; the planar pair fills the whole rectangle
+        self._triangular = not getattr(forward_transform, "_planar", False)
 
     def forward(self, x):
         dtype = x.dtype
@@ -83,7 +86,7 @@ class SpectralConv(nn.Module):
             spec = self.forward_transform.analysis(x if dtype == torch.bfloat16 else x.float())
             if self.scale_residual:
                 residual = self.inverse_transform.synthesis(spec, (B, C), dtype=dtype if dtype == torch.bfloat16 else torch.float32).to(dtype)
-            spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=True, compute=self.compute)
+            spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=self._triangular, compute=self.compute)
             x = self.inverse_transform.synthesis(spec, (B, self.out_channels), dtype=dtype if fuse_cast else torch.float32)
         else:
             x = x.float()

@@ -8,6 +8,16 @@ non-separable dhconv operator without bias.
 import numpy as np
 
 from .sht import sht_forward, sht_inverse
+from .fft2 import Fft2Modes, fft2_forward, fft2_inverse
+
+
+def transform_forward(x, t):
+    """The forward transform `t` describes: spherical tables or the planar pair's mode bookkeeping."""
+    return fft2_forward(x, t) if isinstance(t, Fft2Modes) else sht_forward(x, t)
+
+
+def transform_inverse(c, t):
+    return fft2_inverse(c, t) if isinstance(t, Fft2Modes) else sht_inverse(c, t)
 
 
 def dhconv(x, w):
@@ -38,11 +48,11 @@ def spectral_conv(x, w, fwd_tables, inv_tables, bias=None):
     )
     residual = np.asarray(x, dtype=np.float64)
     contract = diagonal if np.asarray(w).ndim == 4 else dhconv
-    c = sht_forward(x, fwd_tables)
+    c = transform_forward(x, fwd_tables)
     if scale_residual:
-        residual = sht_inverse(c, inv_tables)
+        residual = transform_inverse(c, inv_tables)
     y = contract(c, np.asarray(w, dtype=np.complex128))
-    y = sht_inverse(y, inv_tables)
+    y = transform_inverse(y, inv_tables)
     if bias is not None:
         y = y + bias
     return y, residual

@@ -10,18 +10,25 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .sht import ShtTables, sht_forward, sht_inverse
-from .dhconv import spectral_conv
+from .sht import ShtTables
+from .fft2 import Fft2Modes
+from .dhconv import spectral_conv, transform_forward, transform_inverse
 
 
 class SfnoOracle:
     def __init__(self, inp_shape, out_shape, scale_factor, num_layers, model_grid_type="equiangular", sht_grid_type="legendre-gauss",
-                 activation="gelu", normalization="instance_norm", big_skip=True, use_mlp=True, hard_thresholding_fraction=1.0):
+                 activation="gelu", normalization="instance_norm", big_skip=True, use_mlp=True, hard_thresholding_fraction=1.0,
+                 spectral_transform="sht"):
         h, w = inp_shape[0] // scale_factor, inp_shape[1] // scale_factor
         ml, mm = int(h * hard_thresholding_fraction), int((w // 2 + 1) * hard_thresholding_fraction)
-        self.down = ShtTables(inp_shape[0], inp_shape[1], ml, mm, model_grid_type)
-        self.up = ShtTables(out_shape[0], out_shape[1], ml, mm, model_grid_type)
-        self.mid = ShtTables(h, w, ml, mm, sht_grid_type)
+        if spectral_transform == "fft":      # sfnonet.py:542-556
+            self.down = Fft2Modes(inp_shape[0], inp_shape[1], ml, mm)
+            self.up = Fft2Modes(out_shape[0], out_shape[1], ml, mm)
+            self.mid = Fft2Modes(h, w, ml, mm)
+        else:
+            self.down = ShtTables(inp_shape[0], inp_shape[1], ml, mm, model_grid_type)
+            self.up = ShtTables(out_shape[0], out_shape[1], ml, mm, model_grid_type)
+            self.mid = ShtTables(h, w, ml, mm, sht_grid_type)
         self.inp_shape, self.out_shape = tuple(inp_shape), tuple(out_shape)
         self.num_layers, self.big_skip, self.use_mlp = num_layers, big_skip, use_mlp
         self.act = {"gelu": F.gelu, "relu": F.relu, "silu": F.silu}[activation]
@@ -43,7 +50,7 @@ class SfnoOracle:
         x = x.detach().cpu().double()
         if self.big_skip:
             if self.out_shape != self.inp_shape:
-                residual = torch.from_numpy(sht_inverse(sht_forward(x.numpy(), self.down), self.up))
+                residual = torch.from_numpy(transform_inverse(transform_forward(x.numpy(), self.down), self.up))
             else:
                 residual = x
         y = self._conv(self.act(self._conv(x, sd, "encoder.fwd.0")), sd, "encoder.fwd.2")
@@ -53,7 +60,7 @@ class SfnoOracle:
         elif "pos_embed.0" in sd:
             re, im = sd["pos_embed.0"].double().numpy(), sd["pos_embed.1"].double().numpy()
             c = re + 1j * np.pad(im, ((0, 0), (0, 0), (0, 0), (1, 0)))
-            y = y + torch.from_numpy(sht_inverse(c, self.up))
+            y = y + torch.from_numpy(transform_inverse(c, self.up))
         for i in range(self.num_layers):
             fwd = self.down if i == 0 else self.mid
             inv = self.up if i == self.num_layers - 1 else self.mid

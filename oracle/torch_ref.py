@@ -54,5 +54,33 @@ class TorchRefSHT:
         return torch.fft.irfft(x, n=self.nlon, dim=-1, norm="forward")
 
 
+class TorchRefFFT2:
+    """The torch op sequence of RealFFT2.forward / InverseRealFFT2.forward (makani/models/common/layers.py:242-250,
+    276-287); autograd through it is the gradient oracle of the planar pair."""
+
+    def __init__(self, nlat, nlon, lmax=None, mmax=None):
+        from .fft2 import Fft2Modes
+
+        t = Fft2Modes(nlat, nlon, lmax, mmax)
+        self.nlat, self.nlon, self.lmax, self.mmax, self.truncate = nlat, nlon, t.lmax, t.mmax, t.truncate
+        self.lmax_high, self.lmax_low = t.lmax_high, t.lmax_low
+
+    def forward(self, x):
+        y = torch.fft.rfft2(x, s=(self.nlat, self.nlon), dim=(-2, -1), norm="ortho")
+        if self.truncate:
+            lo = y[..., y.shape[-2] - self.lmax_low :, : self.mmax]
+            y = torch.cat((y[..., : self.lmax_high, : self.mmax], lo), dim=-2)
+        return y
+
+    def inverse(self, c):
+        xt = c[..., : self.mmax]
+        if self.truncate:
+            xth = xt[..., : self.lmax_high, :]
+            xtl = xt[..., xt.shape[-2] - self.lmax_low :, :]
+            xthp = torch.nn.functional.pad(xth, (0, 0, 0, self.nlat - self.lmax))
+            xt = torch.cat([xthp, xtl], dim=-2)
+        return torch.fft.irfft2(xt, s=(self.nlat, self.nlon), dim=(-2, -1), norm="ortho")
+
+
 def dhconv(x, w):
     return torch.einsum("bixy,iox->boxy", x, w)

@@ -257,6 +257,10 @@ def bench_fft2_pair(args):
     def step():
         return inv(fwd(x))
 
+    if args.yardstick:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.mul(src, 1.0)            # reads 256 MiB, writes 256 MiB
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -303,7 +307,8 @@ def bench_fft2_pair(args):
         "data": "synthetic",
         "config": {"workload": "RealFFT2 + InverseRealFFT2 (spectral_transform='fft'), 720x1440, all modes, batch 1, 73 channels, Gaussian random fields"},
         "roofline": {"kernel": f"latfft_kernel ({dom})", "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": gbs / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes_per_launch": lat_bytes, "avg_launch_ms": stage_ms[dom]},
+                     "frac": gbs / PEAK_HBM_GBS, "traffic": read_traffic("fft2_" + dom), "algorithmic_bytes_per_launch": lat_bytes,
+                     "avg_launch_ms": stage_ms[dom]},
         "stages_ms": stage_ms,
     }
     if not args.no_cpu_baseline:

@@ -285,7 +285,8 @@ static const size_t kFftMaxLds = 160 * 1024;
 //            the floor(lmax/2) highest (negative) frequencies n - lmax + j.
 //   INV = 1: k = kept frequency, j = latitude; dropped frequencies are zero.
 // Every output is multiplied by mscale[m] (normalisation, and the order weights of the adjoint transforms).
-// grid = (mmax, ceil(ld / 2 / 2^cshift)); dynamic LDS = 2 * n * 2^cshift * sizeof(float2)
+// grid = (ceil(ld / 2 / 2^cshift), mmax): the channel groups of one order are neighbours in dispatch order;
+// dynamic LDS = 2 * n * 2^cshift * sizeof(float2)
 constexpr int LATFFT_THREADS = 512;
 
 template <int INV>
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(LATFFT_THREADS) void latfft_kernel(FftDev f, const 
                                                                 int cshift, const float* __restrict__ mscale) {
     extern __shared__ __align__(16) float2 lds[];
     const int n = f.n, tid = threadIdx.x, cw = 1 << cshift;
-    const int m = blockIdx.x, c0 = blockIdx.y * cw;
+    const int m = blockIdx.y, c0 = blockIdx.x * cw;
     const int lhigh = (lmax + 1) / 2, gap = n - lmax;
     float2* buf0 = lds;
     float2* buf1 = lds + n * cw;
@@ -337,7 +338,8 @@ int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, i
         attr_set = true;
     }
     const int cw = 1 << cshift;
-    dim3 grid(mmax, (unsigned)((ld / 2 + cw - 1) / cw));
+    if (mmax > 65535) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)((ld / 2 + cw - 1) / cw), mmax);
     if (inverse)
         hipLaunchKernelGGL(latfft_kernel<1>, grid, dim3(LATFFT_THREADS), lds, s, make_dev(p), in, out, lmax, ld, cshift, mscale);
     else

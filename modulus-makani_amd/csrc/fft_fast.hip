@@ -454,16 +454,20 @@ __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict
 // transposed on the way into LDS, where each channel is one sequence of the in-place passes above.
 //   INV = 0: decimation in frequency; kept frequency f leaves from slot pos(f).
 //   INV = 1: decimation in time; kept frequency f enters at slot pos(f), dropped frequencies enter as zeros.
-// grid = (mmax, ceil(ld / 16))
+// grid = 8 * ceil(mmax/8) * ceil(ld / 16) workgroups: all channel groups of one order run back to back on one XCD
+// (map_block), so that the two 64-byte halves of a 128-byte line are fetched into that XCD's L2 once.
 constexpr int LS = 8;
 
 template <int N, int R0, int R1, int R2, int FT, int INV>
 __global__ __launch_bounds__(FT) void latfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ in,
-                                                         float* __restrict__ out, int lmax, int ld, const float* __restrict__ mscale) {
+                                                         float* __restrict__ out, int mmax, int lmax, int ld, int ngroups,
+                                                         const float* __restrict__ mscale) {
     using G = Geo<N, R0, R1, R2>;
     __shared__ __align__(16) float2 z[LS * G::PITCH];
     const int tid = threadIdx.x;
-    const int m = blockIdx.x, c0 = blockIdx.y * LS;
+    int m, group;
+    if (!map_block(mmax, ngroups, m, group)) return;
+    const int c0 = group * LS;
     const int lhigh = (lmax + 1) / 2, gap = N - lmax;
     const int nin = INV ? lmax : N, nout = INV ? N : lmax;
     const int c = tid & (LS - 1);
@@ -536,11 +540,14 @@ int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t r
 template <int N, int R0, int R1, int R2>
 int go_lat(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
     constexpr int FT = (LS * N >= 4096) ? 512 : 256;
-    dim3 grid(mmax, (unsigned)((ld / 2 + LS - 1) / LS));
+    const int ngroups = (ld / 2 + LS - 1) / LS;
+    const int64_t nblocks = (int64_t)((mmax + 7) / 8) * ngroups * 8;
+    if (nblocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)nblocks);
     if (inverse)
-        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 1>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, lmax, ld, mscale);
+        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 1>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, mmax, lmax, ld, ngroups, mscale);
     else
-        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 0>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, lmax, ld, mscale);
+        hipLaunchKernelGGL((latfft_fast_kernel<N, R0, R1, R2, FT, 0>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, out, mmax, lmax, ld, ngroups, mscale);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

@@ -6,13 +6,28 @@
 
 namespace sfno {
 
-// grid (ceil(mmax/32), lmax, ceil(rows/32)), block (32, 8)
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  A tile is 32 orders x 32 rows of one degree; its
+// 256-byte pieces of the reference layout start wherever (r lmax + l) mmax + m0 falls, so neighbouring order tiles
+// share 128-byte lines.  All order tiles of one (degree, row tile) therefore run back to back on one XCD, where
+// the shared lines meet in that XCD's L2; degrees go to the XCDs round-robin.
+// grid = 8 * mtiles * ceil(lmax/8) * rtiles workgroups, block (32, 8)
+__device__ __forceinline__ bool map_tile(int mtiles, int lmax, int& m0, int& l, int64_t& r0) {
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int l8 = (lmax + 7) / 8;
+    const int t = q / mtiles;
+    m0 = (q - t * mtiles) * 32;
+    l = (t % l8) * 8 + xcd;
+    r0 = (int64_t)(t / l8) * 32;
+    return l < lmax;
+}
+
 __global__ __launch_bounds__(256) void spectral_to_coeffs_kernel(const float* __restrict__ spec, float2* __restrict__ coeffs, int64_t rows,
-                                                                 int lmax, int mmax, int ld, int tri) {
+                                                                 int lmax, int mmax, int ld, int tri, int mtiles) {
     __shared__ float2 tile[32][33];
     const int tx = threadIdx.x, ty = threadIdx.y;
-    const int m0 = blockIdx.x * 32, l = blockIdx.y;
-    const int64_t r0 = (int64_t)blockIdx.z * 32;
+    int m0, l;
+    int64_t r0;
+    if (!map_tile(mtiles, lmax, m0, l, r0)) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int mm = ty + 8 * i, m = m0 + mm;
@@ -31,12 +46,13 @@ __global__ __launch_bounds__(256) void spectral_to_coeffs_kernel(const float* __
 }
 
 __global__ __launch_bounds__(256) void coeffs_to_spectral_kernel(const float2* __restrict__ coeffs, float* __restrict__ spec, int64_t rows,
-                                                                 int lmax, int mmax, int ld, int tri) {
+                                                                 int lmax, int mmax, int ld, int tri, int mtiles) {
     __shared__ float2 tile[32][33];
     const int tx = threadIdx.x, ty = threadIdx.y;
-    const int m0 = blockIdx.x * 32, l = blockIdx.y;
+    int m0, l;
+    int64_t r0;
+    if (!map_tile(mtiles, lmax, m0, l, r0)) return;
     if (tri && m0 > l) return;          // a tile entirely above the diagonal holds nothing to move
-    const int64_t r0 = (int64_t)blockIdx.z * 32;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int rr = ty + 8 * i, m = m0 + tx;
@@ -59,20 +75,27 @@ __global__ __launch_bounds__(256) void coeffs_to_spectral_kernel(const float2* _
     }
 }
 
-static bool grid_ok(int64_t rows, int lmax) { return rows > 0 && lmax > 0 && lmax <= 65535 && (rows + 31) / 32 <= 65535; }
+// number of workgroups for `rtiles` row tiles, or 0 if the grid does not fit
+static unsigned tile_blocks(int lmax, int mmax, int64_t rtiles) {
+    if (lmax <= 0 || mmax <= 0 || rtiles <= 0) return 0;
+    const int64_t n = 8 * (int64_t)((mmax + 31) / 32) * ((lmax + 7) / 8) * rtiles;
+    return n > 0x7fffffffLL ? 0 : (unsigned)n;
+}
 
 int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri, hipStream_t s) {
-    if (!grid_ok(rows, lmax) || mmax <= 0 || ld < 2 * rows) return SFNO_EINVAL;
-    // the z range covers the padded channel slots too (ld/2 >= rows)
-    dim3 grid((mmax + 31) / 32, lmax, (unsigned)((ld / 2 + 31) / 32));
-    hipLaunchKernelGGL(coeffs_to_spectral_kernel, grid, dim3(32, 8), 0, s, coeffs, spec, rows, lmax, mmax, ld, tri);
+    if (rows <= 0 || ld < 2 * rows) return SFNO_EINVAL;
+    // the row tiles cover the padded channel slots too (ld/2 >= rows)
+    const unsigned blocks = tile_blocks(lmax, mmax, (ld / 2 + 31) / 32);
+    if (!blocks) return SFNO_EINVAL;
+    hipLaunchKernelGGL(coeffs_to_spectral_kernel, dim3(blocks), dim3(32, 8), 0, s, coeffs, spec, rows, lmax, mmax, ld, tri, (mmax + 31) / 32);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
 int spectral_to_coeffs_launch(const float* spec, float2* coeffs, int64_t rows, int lmax, int mmax, int ld, int tri, hipStream_t s) {
-    if (!grid_ok(rows, lmax) || mmax <= 0 || ld < 2 * rows) return SFNO_EINVAL;
-    dim3 grid((mmax + 31) / 32, lmax, (unsigned)((rows + 31) / 32));
-    hipLaunchKernelGGL(spectral_to_coeffs_kernel, grid, dim3(32, 8), 0, s, spec, coeffs, rows, lmax, mmax, ld, tri);
+    if (rows <= 0 || ld < 2 * rows) return SFNO_EINVAL;
+    const unsigned blocks = tile_blocks(lmax, mmax, (rows + 31) / 32);
+    if (!blocks) return SFNO_EINVAL;
+    hipLaunchKernelGGL(spectral_to_coeffs_kernel, dim3(blocks), dim3(32, 8), 0, s, spec, coeffs, rows, lmax, mmax, ld, tri, (mmax + 31) / 32);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

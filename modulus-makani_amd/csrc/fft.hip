@@ -330,13 +330,11 @@ int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, i
     while (cshift > 0 && (2 * sizeof(float2) * p.n << cshift) > kFftMaxLds) --cshift;
     const size_t lds = 2 * sizeof(float2) * p.n << cshift;
     if (lds > kFftMaxLds) return SFNO_EUNSUPPORTED;
-    static bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)latfft_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess ||
-            hipFuncSetAttribute((const void*)latfft_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess)
-            return SFNO_EHIP;
-        attr_set = true;
-    }
+    // the limit is a property of the function on the current device: set it on every launch that needs it (a host-side call)
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute(inverse ? (const void*)latfft_kernel<1> : (const void*)latfft_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kFftMaxLds) != hipSuccess)
+        return SFNO_EHIP;
     const int cw = 1 << cshift;
     if (mmax > 65535) return SFNO_EUNSUPPORTED;
     dim3 grid((unsigned)((ld / 2 + cw - 1) / cw), mmax);
@@ -350,11 +348,10 @@ int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, i
 template <int PAIRS>
 static int rfft_go(const FftPlan& p, const float* x, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     size_t lds = 2 * (size_t)PAIRS * p.n * sizeof(float2);
-    static bool attr_set = false;
-    if (!attr_set && lds > 64 * 1024) {
-        if (hipFuncSetAttribute((const void*)rfft_kernel<PAIRS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess) return SFNO_EHIP;
-        attr_set = true;
-    }
+    // the limit is a property of the function on the current device: set it on every launch that needs it (a host-side call)
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)rfft_kernel<PAIRS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess)
+        return SFNO_EHIP;
     dim3 grid(nlat, (unsigned)((ld / 4 + PAIRS - 1) / PAIRS));
     float scale = (float)(2.0 * 3.14159265358979323846264338327950288 / (double)p.n);
     hipLaunchKernelGGL((rfft_kernel<PAIRS>), grid, dim3(FFT_THREADS), lds, s, make_dev(p), x, xm, rows, nlat, mmax, ld, scale);
@@ -364,11 +361,10 @@ static int rfft_go(const FftPlan& p, const float* x, float* xm, int64_t rows, in
 template <int PAIRS>
 static int irfft_go(const FftPlan& p, const float* xm, float* x, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
     size_t lds = 2 * (size_t)PAIRS * p.n * sizeof(float2);
-    static bool attr_set = false;
-    if (!attr_set && lds > 64 * 1024) {
-        if (hipFuncSetAttribute((const void*)irfft_kernel<PAIRS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess) return SFNO_EHIP;
-        attr_set = true;
-    }
+    // the limit is a property of the function on the current device: set it on every launch that needs it (a host-side call)
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)irfft_kernel<PAIRS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFftMaxLds) != hipSuccess)
+        return SFNO_EHIP;
     dim3 grid(nlat, (unsigned)((ld / 4 + PAIRS - 1) / PAIRS));
     hipLaunchKernelGGL((irfft_kernel<PAIRS>), grid, dim3(FFT_THREADS), lds, s, make_dev(p), xm, x, rows, nlat, mmax, ld);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;

@@ -255,3 +255,27 @@ def test_full_size_properties(lib_built):
     assert float(torch.linalg.norm((back - x).double().ravel()) / torch.linalg.norm(x.double().ravel())) < TOL
     xb = x.to(torch.bfloat16)
     assert torch.equal(fwd.analysis(xb), fwd.analysis(xb.float()))
+
+
+@pytest.mark.gpu
+def test_planar_plan_argument_checks(lib_built):
+    """A planar plan keeps at most nlat latitude and nlon/2+1 longitude frequencies; the module clamps like the
+    reference (layers.py:233-234), the C entry point rejects."""
+    import ctypes
+
+    import makani_amd as ma
+    from makani_amd import _lib
+
+    h = ctypes.c_void_p()
+    planar, ortho = _lib.GRID["planar"], _lib.NORM["ortho"]
+    assert _lib.lib.sfno_sht_plan_create(16, 32, 17, 17, planar, ortho, 1, _lib.DIR_FORWARD, _lib.COMPUTE_FP32, ctypes.byref(h)) == -1
+    assert _lib.lib.sfno_sht_plan_create(16, 32, 16, 18, planar, ortho, 1, _lib.DIR_INVERSE, _lib.COMPUTE_FP32, ctypes.byref(h)) == -1
+    assert not h.value
+    f = ma.RealFFT2(16, 32, lmax=40, mmax=40)
+    assert (f.lmax, f.mmax) == (16, 17)
+    y = f(torch.ones(2, 16, 32, device="cuda"))
+    torch.cuda.synchronize()
+    # a constant field has a single non-zero coefficient, sqrt(nlat nlon) with the "ortho" normalisation
+    want = torch.zeros(2, 16, 17, dtype=torch.complex64)
+    want[:, 0, 0] = (16 * 32) ** 0.5
+    assert torch.allclose(y.cpu(), want, atol=1e-5)

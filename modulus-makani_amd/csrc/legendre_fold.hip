@@ -285,6 +285,8 @@ template <bool ANALYSIS, int MODE>
 static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     const int64_t ncols = a.ld;
     if (n_work <= 0 || ncols <= 0) return SFNO_OK;
+    // the kernel addresses a panel (one order: nlat or lmax rows of ld floats) with 32-bit byte offsets
+    if ((int64_t)(a.nlat > a.lmax ? a.nlat : a.lmax) * a.ld >= ((int64_t)1 << 30)) return SFNO_EUNSUPPORTED;
     // 4 tiles keep four wavefronts per SIMD resident, 5 three; prefer the least padding, then occupancy
     static const int cand[] = {4, 5, 3, 2, 1};
     int best = 1;

@@ -510,7 +510,8 @@ struct FastEntry {
     int n, r0, r1, r2;
 };
 // lengths with a specialised kernel; the last radix acts on contiguous groups, an odd one keeps LDS banks apart
-const FastEntry kFast[] = {{1440, 16, 10, 9}, {720, 16, 5, 9}, {480, 10, 16, 3}, {240, 16, 5, 3}, {64, 8, 8, 1}, {180, 4, 5, 9}};
+const FastEntry kFast[] = {{1440, 16, 10, 9}, {1024, 16, 8, 8}, {720, 16, 5, 9}, {512, 8, 8, 8}, {480, 10, 16, 3}, {360, 8, 5, 9},
+                           {256, 16, 16, 1}, {240, 16, 5, 3}, {180, 4, 5, 9}, {128, 8, 16, 1}, {64, 8, 8, 1}};
 
 const FastEntry* find_fast(int n) {
     for (const auto& e : kFast)
@@ -557,10 +558,15 @@ bool fft_fast_supported(int n) { return find_fast(n) != nullptr; }
 
 int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
     switch (p.n) {
+        case 1024: return go_lat<1024, 16, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 720: return go_lat<720, 16, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 512: return go_lat<512, 8, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 480: return go_lat<480, 10, 16, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 360: return go_lat<360, 8, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 256: return go_lat<256, 16, 16, 1>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 240: return go_lat<240, 16, 5, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 180: return go_lat<180, 4, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 128: return go_lat<128, 8, 16, 1>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 64: return go_lat<64, 8, 8, 1>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
     }
     return SFNO_EUNSUPPORTED;
@@ -599,11 +605,16 @@ int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, i
                   : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, s);
     switch (p.n) {
         FF_CASE(1440, 16, 10, 9)
+        FF_CASE(1024, 16, 8, 8)
         FF_CASE(720, 16, 5, 9)
+        FF_CASE(512, 8, 8, 8)
         FF_CASE(480, 10, 16, 3)
+        FF_CASE(360, 8, 5, 9)
+        FF_CASE(256, 16, 16, 1)
         FF_CASE(240, 16, 5, 3)
-        FF_CASE(64, 8, 8, 1)
         FF_CASE(180, 4, 5, 9)
+        FF_CASE(128, 8, 16, 1)
+        FF_CASE(64, 8, 8, 1)
     }
 #undef FF_CASE
     return SFNO_EUNSUPPORTED;

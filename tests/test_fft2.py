@@ -258,6 +258,25 @@ def test_full_size_properties(lib_built):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("nlat", [1024, 720, 512, 480, 360, 256, 240, 180, 128, 64])
+def test_every_specialised_latitude_length(lib_built, nlat):
+    """Each latitude length with compile-time passes, truncated and not, against the oracle."""
+    import makani_amd as ma
+
+    print(f"case specialised nlat={nlat}", flush=True)
+    rng = np.random.default_rng(nlat)
+    for lmax in (None, nlat // 3 + 1):
+        t = Fft2Modes(nlat, 24, lmax, None)
+        x = rng.standard_normal((7, nlat, 24)).astype(np.float32)
+        c = (rng.standard_normal((7, t.lmax, t.mmax)) + 1j * rng.standard_normal((7, t.lmax, t.mmax))).astype(np.complex64)
+        y = ma.RealFFT2(nlat, 24, lmax)(torch.from_numpy(x).cuda())
+        z = ma.InverseRealFFT2(nlat, 24, lmax)(torch.from_numpy(c).cuda())
+        torch.cuda.synchronize()
+        assert rel_l2(y.cpu().numpy(), fft2_forward(x.astype(np.float64), t)) < TOL
+        assert rel_l2(z.cpu().numpy(), fft2_inverse(c.astype(np.complex128), t)) < TOL
+
+
+@pytest.mark.gpu
 def test_planar_plan_argument_checks(lib_built):
     """A planar plan keeps at most nlat latitude and nlon/2+1 longitude frequencies; the module clamps like the
     reference (layers.py:233-234), the C entry point rejects."""

@@ -219,3 +219,28 @@ def test_known_answers_config0(lib_built):
     torch.cuda.synchronize()
     assert np.linalg.norm(c.cpu().numpy() - g["forward"]) / np.linalg.norm(g["forward"]) < 1e-5
     assert np.linalg.norm(x.cpu().numpy() - g["inverse"]) / np.linalg.norm(g["inverse"]) < 1e-5
+
+
+@pytest.mark.parametrize("nlon", [1440, 1024, 720, 512, 480, 360, 256, 240, 180, 128, 64])
+def test_every_specialised_longitude_length(lib_built, nlon):
+    """Each transform length with compile-time passes, through the whole pair on a small latitude count: forward and
+    inverse against the oracle, and bf16 grid input equal to its float32 widening."""
+    import makani_amd as ma
+
+    nlat, mmax, lead = 9, min(nlon // 2 + 1, 300), (2, 5)
+    print(f"case specialised nlon={nlon}", flush=True)
+    t = ShtTables(nlat, nlon, nlat, mmax, "legendre-gauss")
+    torch.manual_seed(nlon)
+    x = torch.randn(*lead, nlat, nlon)
+    c = torch.randn(*lead, t.lmax, t.mmax, dtype=torch.complex64)
+    sht = ma.RealSHT(nlat, nlon, lmax=nlat, mmax=mmax, grid="legendre-gauss")
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=nlat, mmax=mmax, grid="legendre-gauss")
+    got_f, got_i = sht(x.cuda()), isht(c.cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(got_f.cpu().numpy(), sht_forward(x.double().numpy(), t)) < TOL
+    assert rel_l2(got_i.cpu().numpy(), sht_inverse(c.numpy().astype(np.complex128), t)) < TOL
+    xb = x.to(torch.bfloat16).cuda()
+    a, b = sht.analysis(xb), sht.analysis(xb.float())
+    m, l = torch.arange(mmax)[:, None], torch.arange(nlat)[None, :]
+    keep = (m <= l).cuda()
+    assert torch.equal(a[..., : 2 * 10][keep], b[..., : 2 * 10][keep])

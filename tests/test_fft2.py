@@ -277,6 +277,25 @@ def test_every_specialised_latitude_length(lib_built, nlat):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("nlat,lmax", [(721, None), (721, 240), (1300, 100)])
+def test_long_latitude_lengths_without_specialised_passes(lib_built, nlat, lmax):
+    """721 = 7 * 103 (the 0.25 degree grid with both poles) and 1300 = 4 * 25 * 13 run on the run-time radix passes
+    with more than 64 KB of LDS per workgroup."""
+    import makani_amd as ma
+
+    print(f"case generic nlat={nlat} lmax={lmax}", flush=True)
+    rng = np.random.default_rng(nlat)
+    t = Fft2Modes(nlat, 16, lmax, None)
+    x = rng.standard_normal((5, nlat, 16)).astype(np.float32)
+    c = (rng.standard_normal((5, t.lmax, t.mmax)) + 1j * rng.standard_normal((5, t.lmax, t.mmax))).astype(np.complex64)
+    y = ma.RealFFT2(nlat, 16, lmax)(torch.from_numpy(x).cuda())
+    z = ma.InverseRealFFT2(nlat, 16, lmax)(torch.from_numpy(c).cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(y.cpu().numpy(), fft2_forward(x.astype(np.float64), t)) < TOL
+    assert rel_l2(z.cpu().numpy(), fft2_inverse(c.astype(np.complex128), t)) < TOL
+
+
+@pytest.mark.gpu
 def test_planar_plan_argument_checks(lib_built):
     """A planar plan keeps at most nlat latitude and nlon/2+1 longitude frequencies; the module clamps like the
     reference (layers.py:233-234), the C entry point rejects."""

@@ -107,6 +107,7 @@ enum { MS_FWD = 0, MS_INV = 1, MS_FWD_ADJ = 2, MS_INV_ADJ = 3 };
 int planar_init(sfno_sht_plan* p) {
     int rc = fft_plan_init(p->fft, p->nlon);
     if (rc == SFNO_OK) rc = fft_plan_init(p->fft_lat, p->nlat);
+    if (rc == SFNO_OK) rc = fft_chirp_plan_init(p->fft_lat);
     if (rc != SFNO_OK) return rc;
     const double s = 2.0 * 3.14159265358979323846264338327950288 / p->nlon;
     const double b = 1.0 / std::sqrt((double)p->nlat * (double)p->nlon), a = b / s;

@@ -262,7 +262,10 @@ void fft_plan_free(FftPlan& p) {
     if (p.d_tw) (void)hipFree(p.d_tw);
     if (p.d_tw0) (void)hipFree(p.d_tw0);
     if (p.d_tw1) (void)hipFree(p.d_tw1);
-    p.d_tw = p.d_tw0 = p.d_tw1 = nullptr;
+    if (p.d_chirp) (void)hipFree(p.d_chirp);
+    if (p.d_vhat) (void)hipFree(p.d_vhat);
+    p.d_tw = p.d_tw0 = p.d_tw1 = p.d_chirp = p.d_vhat = nullptr;
+    p.chirp_m = 0;
 }
 
 static FftDev make_dev(const FftPlan& p) {
@@ -321,7 +324,7 @@ __global__ __launch_bounds__(LATFFT_THREADS) void latfft_kernel(FftDev f, const 
 
 int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
     if (lmax < 1 || lmax > p.n || mmax < 1 || ld % 2 != 0 || !mscale) return SFNO_EINVAL;
-    if (fft_fast_supported(p.n)) {
+    if (fft_fast_supported(p.n) || p.chirp_m) {
         const int rc = latfft_fast_launch(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         if (rc != SFNO_EUNSUPPORTED) return rc;
     }

@@ -506,11 +506,53 @@ __global__ __launch_bounds__(FT) void latfft_fast_kernel(const float2* __restric
     }
 }
 
+// Latitude FFT of a length n with a large prime factor (721 = 7 * 103, the 0.25 degree grid with both poles), as a
+// circular convolution of length M >= 2n - 1 on the specialised passes (Bluestein):
+//     X[j] = c[j] sum_k (x[k] c[k]) conj(c)[j - k],   c[k] = exp(-i pi k^2 / n)          (forward; conjugate c for the inverse)
+// u = x c zero-padded to M -> decimation-in-frequency passes -> times vhat (the transform of conj(c) wrapped around M, in
+// the slot order those passes leave, 1/M folded in; conj(c) is even, so the inverse uses conj(vhat)) -> decimation-in-time
+// passes -> times c.  Same layouts, truncation rule and workgroup order as latfft_fast_kernel; S channels per workgroup.
+template <int M, int R0, int R1, int R2, int S, int FT, int INV>
+__global__ __launch_bounds__(FT) void latfft_chirp_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float2* __restrict__ chirp,
+                                                          const float2* __restrict__ vhat, const float* __restrict__ in, float* __restrict__ out, int n,
+                                                          int mmax, int lmax, int ld, int ngroups, const float* __restrict__ mscale) {
+    using G = Geo<M, R0, R1, R2>;
+    __shared__ __align__(16) float2 z[S * G::PITCH];
+    const int tid = threadIdx.x;
+    int m, group;
+    if (!map_block(mmax, ngroups, m, group)) return;
+    const int c0 = group * S;
+    const int lhigh = (lmax + 1) / 2, gap = n - lmax;
+    const int nin = INV ? lmax : n, nout = INV ? n : lmax;
+    const int c = tid & (S - 1);
+    const bool live = 2 * (c0 + c) < ld;
+    const float* src = in + (int64_t)m * nin * ld + 2 * (c0 + c);
+    for (int i = tid / S; i < M; i += FT / S) {
+        const int k = i >= n ? -1 : !INV ? i : i < lhigh ? i : i >= lhigh + gap ? i - gap : -1;
+        float2 v = make_float2(0.f, 0.f);
+        if (k >= 0 && live) v = cmul_tw<INV>(*reinterpret_cast<const float2*>(src + (int64_t)k * ld), chirp[i]);
+        z[c * G::PITCH + i] = v;
+    }
+    __syncthreads();
+    passes_dif<M, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
+    for (int i = tid / S; i < M; i += FT / S) z[c * G::PITCH + i] = cmul_tw<INV>(z[c * G::PITCH + i], vhat[i]);
+    __syncthreads();
+    passes_dit<M, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
+    if (!live) return;
+    const float sc = mscale[m];
+    float* dst = out + (int64_t)m * nout * ld + 2 * (c0 + c);
+    for (int j = tid / S; j < nout; j += FT / S) {
+        const int i = INV ? j : j < lhigh ? j : j + gap;
+        const float2 v = cmul_tw<INV>(z[c * G::PITCH + i], chirp[i]);
+        *reinterpret_cast<float2*>(dst + (int64_t)j * ld) = make_float2(sc * v.x, sc * v.y);
+    }
+}
+
 struct FastEntry {
     int n, r0, r1, r2;
 };
 // lengths with a specialised kernel; the last radix acts on contiguous groups, an odd one keeps LDS banks apart
-const FastEntry kFast[] = {{1440, 16, 10, 9}, {1024, 16, 8, 8}, {720, 16, 5, 9}, {512, 8, 8, 8}, {480, 10, 16, 3}, {360, 8, 5, 9},
+const FastEntry kFast[] = {{1536, 16, 12, 8}, {1440, 16, 10, 9}, {1024, 16, 8, 8}, {720, 16, 5, 9}, {512, 8, 8, 8}, {480, 10, 16, 3}, {360, 8, 5, 9},
                            {256, 16, 16, 1}, {240, 16, 5, 3}, {180, 4, 5, 9}, {128, 8, 16, 1}, {64, 8, 8, 1}};
 
 const FastEntry* find_fast(int n) {
@@ -552,11 +594,100 @@ int go_lat(bool inverse, const FftPlan& p, const float* in, float* out, int mmax
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
+template <int M, int R0, int R1, int R2>
+int go_chirp(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
+    constexpr int S = (M >= 1024) ? 4 : 8;
+    constexpr int FT = 256;
+    const int ngroups = (ld / 2 + S - 1) / S;
+    const int64_t nblocks = (int64_t)((mmax + 7) / 8) * ngroups * 8;
+    if (nblocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    dim3 grid((unsigned)nblocks);
+    if (inverse)
+        hipLaunchKernelGGL((latfft_chirp_kernel<M, R0, R1, R2, S, FT, 1>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, p.d_chirp, p.d_vhat, in, out, p.n, mmax,
+                           lmax, ld, ngroups, mscale);
+    else
+        hipLaunchKernelGGL((latfft_chirp_kernel<M, R0, R1, R2, S, FT, 0>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, p.d_chirp, p.d_vhat, in, out, p.n, mmax,
+                           lmax, ld, ngroups, mscale);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+// inter-pass twiddles of the specialised passes of length f.n
+int upload_pass_twiddles(const FastEntry& f, FftPlan& p) {
+    const int N = f.n, nb = N / f.r0;
+    std::vector<float2> tw0((size_t)(f.r0 - 1) * nb), tw1((size_t)std::max(1, (f.r1 - 1) * f.r2));
+    for (int k0 = 1; k0 < f.r0; ++k0)
+        for (int j = 0; j < nb; ++j) {
+            double a = -kTwoPi * (double)(((int64_t)k0 * j) % N) / (double)N;
+            tw0[(size_t)(k0 - 1) * nb + j] = make_float2((float)std::cos(a), (float)std::sin(a));
+        }
+    tw1[0] = make_float2(1.f, 0.f);
+    for (int k1 = 1; k1 < f.r1; ++k1)
+        for (int n2 = 0; n2 < f.r2; ++n2) {
+            double a = -kTwoPi * (double)(((int64_t)f.r0 * k1 * n2) % N) / (double)N;
+            tw1[(size_t)(k1 - 1) * f.r2 + n2] = make_float2((float)std::cos(a), (float)std::sin(a));
+        }
+    if (hipMalloc(&p.d_tw0, sizeof(float2) * tw0.size()) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMalloc(&p.d_tw1, sizeof(float2) * tw1.size()) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMemcpy(p.d_tw0, tw0.data(), sizeof(float2) * tw0.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
+    if (hipMemcpy(p.d_tw1, tw1.data(), sizeof(float2) * tw1.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
+    return SFNO_OK;
+}
+
+int largest_prime_factor(int n) {
+    int best = 1;
+    for (int q = 2; (int64_t)q * q <= n; ++q)
+        while (n % q == 0) { best = q; n /= q; }
+    return n > 1 ? n : best;
+}
+
 }  // namespace
 
 bool fft_fast_supported(int n) { return find_fast(n) != nullptr; }
 
+int fft_chirp_plan_init(FftPlan& p) {
+    const int n = p.n;
+    if (find_fast(n) || largest_prime_factor(n) <= 7) return SFNO_OK;      // the plain passes serve these lengths well
+    const int M = 2 * n - 1 <= 512 ? 512 : 2 * n - 1 <= 1536 ? 1536 : 0;
+    if (!M) return SFNO_OK;
+    const FastEntry* f = find_fast(M);
+    // chirp c[k] = exp(-i pi k^2 / n), the angle reduced exactly in integers
+    std::vector<double> cr(n), ci(n);
+    std::vector<float2> chirp(M, make_float2(0.f, 0.f));
+    for (int k = 0; k < n; ++k) {
+        const double a = -(kTwoPi / 2) * (double)(((int64_t)k * k) % (2 * (int64_t)n)) / (double)n;
+        cr[k] = std::cos(a);
+        ci[k] = std::sin(a);
+        chirp[k] = make_float2((float)cr[k], (float)ci[k]);
+    }
+    // v = conj(c) wrapped around M (v[M - k] = v[k]); its transform, real-symmetric input pairs folded:
+    // V[q] = v[0] + sum_{k=1}^{n-1} v[k] 2 cos(2 pi q k / M)
+    std::vector<float2> vhat(M);
+    std::vector<double> cosM(M);
+    for (int j = 0; j < M; ++j) cosM[j] = std::cos(kTwoPi * (double)j / (double)M);
+    const int r0 = f->r0, r1 = f->r1, r2 = f->r2;
+    for (int q = 0; q < M; ++q) {
+        double sr = cr[0], si = -ci[0];
+        for (int k = 1; k < n; ++k) {
+            const double w = 2.0 * cosM[(int)(((int64_t)q * k) % M)];
+            sr += cr[k] * w;
+            si -= ci[k] * w;
+        }
+        const int k0 = q % r0, t = q / r0, k1 = t % r1, k2 = t / r1;        // slot of bin q after the decimation-in-frequency passes
+        vhat[k0 * (r1 * r2) + k1 * r2 + k2] = make_float2((float)(sr / M), (float)(si / M));
+    }
+    int rc = upload_pass_twiddles(*f, p);
+    if (rc != SFNO_OK) return rc;
+    if (hipMalloc(&p.d_chirp, sizeof(float2) * M) != hipSuccess || hipMalloc(&p.d_vhat, sizeof(float2) * M) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMemcpy(p.d_chirp, chirp.data(), sizeof(float2) * M, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(p.d_vhat, vhat.data(), sizeof(float2) * M, hipMemcpyHostToDevice) != hipSuccess)
+        return SFNO_EHIP;
+    p.chirp_m = M;
+    return SFNO_OK;
+}
+
 int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s) {
+    if (p.chirp_m == 1536) return go_chirp<1536, 16, 12, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+    if (p.chirp_m == 512) return go_chirp<512, 8, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
     switch (p.n) {
         case 1024: return go_lat<1024, 16, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 720: return go_lat<720, 16, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
@@ -574,25 +705,7 @@ int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* o
 
 int fft_fast_plan_init(FftPlan& p) {
     const FastEntry* f = find_fast(p.n);
-    if (!f) return SFNO_OK;
-    const int N = f->n, nb = N / f->r0;
-    std::vector<float2> tw0((size_t)(f->r0 - 1) * nb), tw1((size_t)std::max(1, (f->r1 - 1) * f->r2));
-    for (int k0 = 1; k0 < f->r0; ++k0)
-        for (int j = 0; j < nb; ++j) {
-            double a = -kTwoPi * (double)(((int64_t)k0 * j) % N) / (double)N;
-            tw0[(size_t)(k0 - 1) * nb + j] = make_float2((float)std::cos(a), (float)std::sin(a));
-        }
-    tw1[0] = make_float2(1.f, 0.f);
-    for (int k1 = 1; k1 < f->r1; ++k1)
-        for (int n2 = 0; n2 < f->r2; ++n2) {
-            double a = -kTwoPi * (double)(((int64_t)f->r0 * k1 * n2) % N) / (double)N;
-            tw1[(size_t)(k1 - 1) * f->r2 + n2] = make_float2((float)std::cos(a), (float)std::sin(a));
-        }
-    if (hipMalloc(&p.d_tw0, sizeof(float2) * tw0.size()) != hipSuccess) return SFNO_ENOMEM;
-    if (hipMalloc(&p.d_tw1, sizeof(float2) * tw1.size()) != hipSuccess) return SFNO_ENOMEM;
-    if (hipMemcpy(p.d_tw0, tw0.data(), sizeof(float2) * tw0.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
-    if (hipMemcpy(p.d_tw1, tw1.data(), sizeof(float2) * tw1.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
-    return SFNO_OK;
+    return f ? upload_pass_twiddles(*f, p) : SFNO_OK;
 }
 
 int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
@@ -604,6 +717,7 @@ int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, i
         return bf ? go_fast<N_, A_, B_, C_, true>(inverse, p, in, out, rows, nlat, mmax, ld, s)           \
                   : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, s);
     switch (p.n) {
+        FF_CASE(1536, 16, 12, 8)
         FF_CASE(1440, 16, 10, 9)
         FF_CASE(1024, 16, 8, 8)
         FF_CASE(720, 16, 5, 9)

@@ -128,6 +128,11 @@ struct FftPlan {
     float2* d_tw = nullptr;        // [n] exp(-2 pi i j / n)
     float2* d_tw0 = nullptr;       // inter-pass twiddles of the specialised kernels (fft_fast.hip)
     float2* d_tw1 = nullptr;
+    // latitude plans of lengths with a large prime factor (fft_chirp_plan_init): the DFT as a circular convolution of
+    // length chirp_m with a chirp; d_tw0 / d_tw1 then belong to the specialised passes of length chirp_m
+    int chirp_m = 0;
+    float2* d_chirp = nullptr;     // [n] exp(-i pi k^2 / n)
+    float2* d_vhat = nullptr;      // [chirp_m] transform of the conjugate chirp, in the slot order of the passes, divided by chirp_m
 };
 bool fft_fast_supported(int n);
 int fft_fast_plan_init(FftPlan& p);
@@ -137,6 +142,8 @@ int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, i
 // latitude FFT on the specialised passes; SFNO_EUNSUPPORTED for a length without them
 int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s);
 int fft_plan_init(FftPlan& p, int n);
+// adds the chirp tables to a latitude plan whose length has no specialised passes and a prime factor above 7 (no-op otherwise)
+int fft_chirp_plan_init(FftPlan& p);
 void fft_plan_free(FftPlan& p);
 // x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon
 int rfft_launch(const FftPlan& p, const void* x, int x_dtype, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);

@@ -221,7 +221,7 @@ def test_known_answers_config0(lib_built):
     assert np.linalg.norm(x.cpu().numpy() - g["inverse"]) / np.linalg.norm(g["inverse"]) < 1e-5
 
 
-@pytest.mark.parametrize("nlon", [1440, 1024, 720, 512, 480, 360, 256, 240, 180, 128, 64])
+@pytest.mark.parametrize("nlon", [1536, 1440, 1024, 720, 512, 480, 360, 256, 240, 180, 128, 64])
 def test_every_specialised_longitude_length(lib_built, nlon):
     """Each transform length with compile-time passes, through the whole pair on a small latitude count: forward and
     inverse against the oracle, and bf16 grid input equal to its float32 widening."""

@@ -122,6 +122,16 @@ int64_t sfno_spectral_elems(const sfno_sht_plan* plan, int64_t rows);
 /* bytes of scratch the calls below need for `rows` rows */
 size_t sfno_sht_workspace_bytes(const sfno_sht_plan* plan, int64_t rows);
 
+/* sfno_sht_synthesis that also returns, for every channel row and latitude, two moments of the field it writes:
+ * lat_stats float32 [rows][nlat][2] = (mean over longitude, mean over longitude of the squared deviation from that
+ * mean).  They come from the Fourier coefficients the longitude kernel has in hand (mean = Re X_0, deviation =
+ * 2 sum_{0<m<nlon/2} |X_m|^2 + (Re X_{nlon/2})^2) and save the statistics pass of the nn.InstanceNorm2d that
+ * follows SpectralConv in the SFNO block (makani/models/networks/sfnonet.py:246-250); they describe the field before
+ * any rounding to x_dtype.  Only plans whose nlon has specialised kernels (sfno_sht_lat_stats_supported). */
+int sfno_sht_lat_stats_supported(const sfno_sht_plan* plan);
+int sfno_sht_synthesis_lat_stats(const sfno_sht_plan* plan, const float* spec, void* x, int x_dtype, int64_t rows, void* workspace,
+                                 size_t workspace_bytes, float* lat_stats, void* stream);
+
 /* RealSHT.forward: x float32 [rows][nlat][nlon] -> coeffs complex64 [rows][lmax][mmax] */
 int sfno_sht_forward(const sfno_sht_plan* plan, const float* x, void* coeffs, int64_t rows,
                      void* workspace, size_t workspace_bytes, void* stream);
@@ -268,6 +278,11 @@ size_t sfno_instance_norm_workspace_bytes(int64_t rows, int64_t P);
 int sfno_instance_norm_coeffs(const void* x, const float* gamma, const float* beta, float* scale, float* shift,
                               int64_t rows, int channels, int64_t P, float eps, void* workspace,
                               size_t workspace_bytes, void* stream);
+/* The coefficients of sfno_instance_norm_coeffs from the per-latitude moments of sfno_sht_synthesis_lat_stats:
+ * mean = avg_k a_k, biased variance = avg_k ((a_k - mean)^2 + d_k) over the nlat rows (every row has nlon points). */
+int sfno_instance_norm_coeffs_lat(const float* lat_stats, const float* gamma, const float* beta, float* scale, float* shift, int64_t rows,
+                                  int channels, int nlat, float eps, void* stream);
+
 /* y = act(scale[row] * x + shift[row]) on bf16 rows of P pixels: the norm0 -> activation step of
  * sfnonet.py:246-251 once the coefficients above are known. */
 int sfno_scale_shift_act(const void* x, const float* scale, const float* shift, void* y, int64_t rows, int64_t P,

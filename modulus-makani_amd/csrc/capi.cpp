@@ -294,6 +294,21 @@ extern "C" int sfno_sht_synthesis(const sfno_sht_plan* p, const float* spec, voi
     return sfno_irfft(p, w.xm, x, x_dtype, rows, stream);
 }
 
+extern "C" int sfno_sht_lat_stats_supported(const sfno_sht_plan* p) { return p && fft_fast_supported(p->nlon) ? 1 : 0; }
+
+extern "C" int sfno_sht_synthesis_lat_stats(const sfno_sht_plan* p, const float* spec, void* x, int x_dtype, int64_t rows, void* workspace,
+                                            size_t workspace_bytes, float* lat_stats, void* stream) {
+    if (!p || !x || !spec || !lat_stats || !rows_ok(rows)) return SFNO_EINVAL;
+    if (!(p->directions & SFNO_DIR_INVERSE)) return SFNO_EINVAL;
+    if (!sfno_sht_lat_stats_supported(p)) return SFNO_EUNSUPPORTED;
+    Ws w = carve(p, rows, workspace);
+    if (!workspace || workspace_bytes < w.bytes) return SFNO_EWORKSPACE;
+    int rc = sfno_legendre_synthesis(p, spec, w.xm, rows, stream);
+    if (rc != SFNO_OK) return rc;
+    return irfft_launch(p->fft, w.xm, x, x_dtype, rows, p->nlat, p->mmax, (int)sfno_spectral_ld(rows), (hipStream_t)stream,
+                        reinterpret_cast<float2*>(lat_stats));
+}
+
 extern "C" int sfno_sht_forward(const sfno_sht_plan* p, const float* x, void* coeffs, int64_t rows, void* workspace,
                                 size_t workspace_bytes, void* stream) {
     if (!p || !coeffs || !rows_ok(rows)) return SFNO_EINVAL;
@@ -569,6 +584,13 @@ extern "C" int sfno_instance_norm_coeffs(const void* x, const float* gamma, cons
     if (!workspace || workspace_bytes < sfno_instance_norm_workspace_bytes(rows, P)) return SFNO_EWORKSPACE;
     return instance_norm_coeffs_launch(reinterpret_cast<const unsigned short*>(x), gamma, beta, scale, shift, reinterpret_cast<float2*>(workspace),
                                        rows, channels, P, eps, (hipStream_t)stream);
+}
+
+extern "C" int sfno_instance_norm_coeffs_lat(const float* lat_stats, const float* gamma, const float* beta, float* scale, float* shift, int64_t rows,
+                                             int channels, int nlat, float eps, void* stream) {
+    if (!lat_stats || !scale || !shift) return SFNO_EINVAL;
+    return instance_norm_coeffs_lat_launch(reinterpret_cast<const float2*>(lat_stats), gamma, beta, scale, shift, rows, channels, nlat, eps,
+                                           (hipStream_t)stream);
 }
 
 extern "C" int sfno_scale_shift_act(const void* x, const float* scale, const float* shift, void* y, int64_t rows, int64_t P, int act,

@@ -395,10 +395,11 @@ int rfft_launch(const FftPlan& p, const void* xv, int x_dtype, float* xm, int64_
     return SFNO_EUNSUPPORTED;
 }
 
-int irfft_launch(const FftPlan& p, const float* xm, void* xv, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+int irfft_launch(const FftPlan& p, const float* xm, void* xv, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s, float2* lat_stats) {
     // orders above nlon/2 are dropped, as torch.fft.irfft(n=nlon) drops surplus input bins
     if (ld % 4 != 0 || ld < 2 * rows) return SFNO_EINVAL;
-    if (fft_fast_supported(p.n)) return fft_fast_launch(true, p, xm, xv, rows, nlat, mmax, ld, x_dtype, s);
+    if (fft_fast_supported(p.n)) return fft_fast_launch(true, p, xm, xv, rows, nlat, mmax, ld, x_dtype, s, lat_stats);
+    if (lat_stats) return SFNO_EUNSUPPORTED;                      // only the specialised kernels produce the moments
     if (x_dtype != SFNO_DTYPE_F32) return SFNO_EUNSUPPORTED;
     float* x = reinterpret_cast<float*>(xv);
     switch (pick_pairs(p.n)) {

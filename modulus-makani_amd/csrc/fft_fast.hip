@@ -387,11 +387,17 @@ __global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict_
 
 template <int N, int R0, int R1, int R2, int S, int FT, bool BF16>
 __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ xm,
-                                                        void* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups) {
+                                                        void* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups,
+                                                        float2* __restrict__ lat_stats) {
     using G = Geo<N, R0, R1, R2>;
     static_assert(N % 2 == 0, "even length");
+    static_assert(FT % S == 0 && 64 % S == 0, "a thread serves one channel pair");
     __shared__ __align__(16) float2 z[S * G::PITCH];
+    __shared__ float4 red[FT / 64][S];
     const int tid = threadIdx.x;
+    // moments of the output row over longitude, from the coefficients on their way in (lat_stats != null): the mean is
+    // Re X_0, the mean squared deviation from it 2 sum_{0<m<N/2} |X_m|^2 + (Re X_{N/2})^2; (A, B) = the two channels of the pair
+    float mean_a = 0.f, mean_b = 0.f, dev_a = 0.f, dev_b = 0.f;
     int lat, group;
     if (!map_block(nlat, ngroups, lat, group)) return;
     const int pair0 = group * S;
@@ -421,15 +427,46 @@ __global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict
                     float2* zz = z + p * G::PITCH;
                     if (m == 0 || m == HALF) {
                         zz[G::pos(m)] = make_float2(w.x, w.z);                     // C2R: Im of mean and Nyquist bins dropped
+                        if (m == 0) {
+                            mean_a = w.x;
+                            mean_b = w.z;
+                        } else {
+                            dev_a = fmaf(w.x, w.x, dev_a);
+                            dev_b = fmaf(w.z, w.z, dev_b);
+                        }
                     } else {
                         zz[G::pos(m)] = make_float2(w.x - w.w, w.y + w.z);
                         zz[G::pos(N - m)] = make_float2(w.x + w.w, w.z - w.y);
+                        dev_a += 2.f * fmaf(w.x, w.x, w.y * w.y);
+                        dev_b += 2.f * fmaf(w.z, w.z, w.w * w.w);
                     }
                 }
             }
         }
     }
+    if (lat_stats) {
+        // lanes S apart serve the same pair: fold them, one entry per wavefront and pair
+#pragma unroll
+        for (int off = S; off < 64; off <<= 1) {
+            mean_a += __shfl_xor(mean_a, off, 64);
+            mean_b += __shfl_xor(mean_b, off, 64);
+            dev_a += __shfl_xor(dev_a, off, 64);
+            dev_b += __shfl_xor(dev_b, off, 64);
+        }
+        if ((tid & 63) < S) red[tid >> 6][tid & 63] = make_float4(mean_a, mean_b, dev_a, dev_b);
+    }
     __syncthreads();
+    if (lat_stats && tid < S) {
+        float4 t = red[0][tid];
+#pragma unroll
+        for (int w = 1; w < FT / 64; ++w) {
+            const float4 u = red[w][tid];
+            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
+        const int64_t r0 = 2 * (int64_t)(pair0 + tid);
+        if (r0 < rows) lat_stats[r0 * nlat + lat] = make_float2(t.x, t.z);
+        if (r0 + 1 < rows) lat_stats[(r0 + 1) * nlat + lat] = make_float2(t.y, t.w);
+    }
     passes_dit<N, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
     {
         constexpr int Q = N / 4, TOT = S * Q;
@@ -562,7 +599,7 @@ const FastEntry* find_fast(int n) {
 }
 
 template <int N, int R0, int R1, int R2, bool BF16>
-int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, hipStream_t s) {
+int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, float2* lat_stats, hipStream_t s) {
     constexpr int S = (N >= 1024) ? 4 : 8;
     constexpr int FT = (S * N >= 4096) ? 512 : 256;     // threads per workgroup
     const int ngroups = (ld / 4 + S - 1) / S;
@@ -575,7 +612,7 @@ int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t r
                            rows, nlat, mmax, ld, ngroups, scale);
     } else {
         hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, reinterpret_cast<const float*>(in), out,
-                           rows, nlat, mmax, ld, ngroups);
+                           rows, nlat, mmax, ld, ngroups, lat_stats);
     }
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
@@ -709,13 +746,14 @@ int fft_fast_plan_init(FftPlan& p) {
 }
 
 int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
-                    hipStream_t s) {
+                    hipStream_t s, float2* lat_stats) {
     const bool bf = grid_dtype == SFNO_DTYPE_BF16;
     if (!bf && grid_dtype != SFNO_DTYPE_F32) return SFNO_EUNSUPPORTED;
-#define FF_CASE(N_, A_, B_, C_)                                                                          \
-    case N_:                                                                                             \
-        return bf ? go_fast<N_, A_, B_, C_, true>(inverse, p, in, out, rows, nlat, mmax, ld, s)           \
-                  : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, s);
+    if (lat_stats && !inverse) return SFNO_EINVAL;
+#define FF_CASE(N_, A_, B_, C_)                                                                                     \
+    case N_:                                                                                                        \
+        return bf ? go_fast<N_, A_, B_, C_, true>(inverse, p, in, out, rows, nlat, mmax, ld, lat_stats, s)           \
+                  : go_fast<N_, A_, B_, C_, false>(inverse, p, in, out, rows, nlat, mmax, ld, lat_stats, s);
     switch (p.n) {
         FF_CASE(1536, 16, 12, 8)
         FF_CASE(1440, 16, 10, 9)

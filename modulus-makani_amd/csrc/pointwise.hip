@@ -481,6 +481,36 @@ __global__ void row_stats_finalize_kernel(const unsigned short* __restrict__ x, 
     shift[row] = (beta ? beta[c] : 0.f) - mean * sc;
 }
 
+// The same coefficients from per-latitude moments of the field (the inverse longitude kernel's by-product):
+// stats[row][k] = (a_k, d_k), the mean over longitude of latitude row k and of its squared deviation from a_k.
+// mean = avg_k a_k, variance = avg_k ((a_k - mean)^2 + d_k); one wavefront per row, sums in double.
+__global__ __launch_bounds__(64) void lat_stats_finalize_kernel(const float2* __restrict__ stats, const float* __restrict__ gamma,
+                                                                const float* __restrict__ beta, float* __restrict__ scale, float* __restrict__ shift,
+                                                                int channels, int nlat, float eps) {
+    const int64_t row = blockIdx.x;
+    const float2* __restrict__ sr = stats + row * nlat;
+    double s = 0.0;
+    for (int k = threadIdx.x; k < nlat; k += 64) s += (double)sr[k].x;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const double mean = s / nlat;
+    double v = 0.0;
+    for (int k = threadIdx.x; k < nlat; k += 64) {
+        const float2 t = sr[k];
+        const double d = (double)t.x - mean;
+        v += d * d + (double)t.y;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (threadIdx.x == 0) {
+        const float rstd = (float)(1.0 / sqrt(v / nlat + (double)eps));
+        const int c = (int)(row % channels);
+        const float sc = (gamma ? gamma[c] : 1.f) * rstd;
+        scale[row] = sc;
+        shift[row] = (beta ? beta[c] : 0.f) - (float)mean * sc;
+    }
+}
+
 // y = act(scale[row] * x + shift[row]), bf16 -> bf16, 8 pixels per thread
 __global__ __launch_bounds__(256) void scale_shift_act_kernel(const unsigned short* __restrict__ x, const float* __restrict__ scale,
                                                               const float* __restrict__ shift, unsigned short* __restrict__ y, int64_t P,
@@ -556,6 +586,13 @@ int instance_norm_coeffs_launch(const unsigned short* x, const float* gamma, con
     hipLaunchKernelGGL(row_stats_partial_kernel, dim3((unsigned)rows, (unsigned)nseg), dim3(ST_THREADS), 0, s, x, partial, P, nseg);
     hipLaunchKernelGGL(row_stats_finalize_kernel, dim3((unsigned)((rows + 127) / 128)), dim3(128), 0, s, x, partial, gamma, beta, scale, shift, rows,
                        channels, P, nseg, eps);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+int instance_norm_coeffs_lat_launch(const float2* stats, const float* gamma, const float* beta, float* scale, float* shift, int64_t rows, int channels,
+                                    int nlat, float eps, hipStream_t s) {
+    if (rows < 1 || rows > 0x7fffffffLL || channels < 1 || nlat < 1) return SFNO_EINVAL;
+    hipLaunchKernelGGL(lat_stats_finalize_kernel, dim3((unsigned)rows), dim3(64), 0, s, stats, gamma, beta, scale, shift, channels, nlat, eps);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

@@ -92,6 +92,8 @@ int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, 
 int row_stats_segments(int64_t rows, int64_t P);
 int instance_norm_coeffs_launch(const unsigned short* x, const float* gamma, const float* beta, float* scale, float* shift, float2* partial,
                                 int64_t rows, int channels, int64_t P, float eps, hipStream_t s);
+int instance_norm_coeffs_lat_launch(const float2* stats, const float* gamma, const float* beta, float* scale, float* shift, int64_t rows, int channels,
+                                    int nlat, float eps, hipStream_t s);
 int scale_shift_act_launch(const unsigned short* x, const float* scale, const float* shift, unsigned short* y, int64_t rows, int64_t P, int act,
                            hipStream_t s);
 
@@ -137,8 +139,9 @@ struct FftPlan {
 bool fft_fast_supported(int n);
 int fft_fast_plan_init(FftPlan& p);
 // grid_dtype: element type of the grid-side tensor (SFNO_DTYPE_*); the Fourier side is always float
+// lat_stats (inverse only, may be null): float2 [rows][nlat] = mean over longitude of the output row and of its squared deviation from that mean
 int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, int grid_dtype,
-                    hipStream_t s);
+                    hipStream_t s, float2* lat_stats = nullptr);
 // latitude FFT on the specialised passes; SFNO_EUNSUPPORTED for a length without them
 int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s);
 int fft_plan_init(FftPlan& p, int n);
@@ -148,7 +151,7 @@ void fft_plan_free(FftPlan& p);
 // x [rows][nlat][nlon] -> xm [mmax][nlat][ld] (re,im of row r at 2r,2r+1), scaled by 2 pi / nlon
 int rfft_launch(const FftPlan& p, const void* x, int x_dtype, float* xm, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
 // xm [mmax][nlat][ld] -> x [rows][nlat][nlon]
-int irfft_launch(const FftPlan& p, const float* xm, void* x, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s);
+int irfft_launch(const FftPlan& p, const float* xm, void* x, int x_dtype, int64_t rows, int nlat, int mmax, int ld, hipStream_t s, float2* lat_stats = nullptr);
 // latitude FFT of the planar transforms on the order-major layout: in[m][nlat | lmax][ld] -> out[m][lmax | nlat][ld]
 // (forward keeps lmax frequencies, inverse zero-fills the dropped ones); outputs are multiplied by mscale[m] (device array)
 int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, int mmax, int lmax, int ld, const float* mscale, hipStream_t s);

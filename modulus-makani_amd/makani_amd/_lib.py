@@ -47,6 +47,8 @@ def _load():
         "sfno_sht_io_dtype_supported": (i32, [vp, i32]),
         "sfno_sht_analysis": (i32, [vp, vp, i32, vp, i64, vp, sz, vp]),
         "sfno_sht_synthesis": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),
+        "sfno_sht_lat_stats_supported": (i32, [vp]),
+        "sfno_sht_synthesis_lat_stats": (i32, [vp, vp, vp, i32, i64, vp, sz, vp, vp]),
         "sfno_sht_forward_adjoint": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_inverse_adjoint": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_analysis_adjoint": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),
@@ -75,6 +77,7 @@ def _load():
         "sfno_pointwise_conv": (i32, [vp, vp, vp, vp, i32, i32, i32, i64, i32, vp, vp, vp, vp]),
         "sfno_instance_norm_workspace_bytes": (sz, [i64, i64]),
         "sfno_instance_norm_coeffs": (i32, [vp, vp, vp, vp, vp, i64, i32, i64, c.c_float, vp, sz, vp]),
+        "sfno_instance_norm_coeffs_lat": (i32, [vp, vp, vp, vp, vp, i64, i32, i32, c.c_float, vp]),
         "sfno_scale_shift_act": (i32, [vp, vp, vp, vp, i64, i64, i32, vp]),
     }
     for name, (res, args) in sig.items():

@@ -98,6 +98,19 @@ def instance_norm_coeffs(x, gamma=None, beta=None, eps=1e-5):
     return scale, shift
 
 
+def instance_norm_coeffs_lat(lat_stats, batch, gamma=None, beta=None, eps=1e-5):
+    """(scale, shift) float32 [B, C] from the per-latitude moments [B*C, nlat, 2] that InverseRealSHT.synthesis_with_lat_stats returns."""
+    rows, nlat, _ = lat_stats.shape
+    C = rows // batch
+    scale = torch.empty((batch, C), dtype=torch.float32, device=lat_stats.device)
+    shift = torch.empty_like(scale)
+    g = gamma.detach().float().contiguous() if gamma is not None else None
+    b = beta.detach().float().contiguous() if beta is not None else None
+    check(lib.sfno_instance_norm_coeffs_lat(_ptr(lat_stats), _ptr(g), _ptr(b), _ptr(scale), _ptr(shift), rows, C, nlat, float(eps),
+                                            _stream(lat_stats.device)), "sfno_instance_norm_coeffs_lat")
+    return scale, shift
+
+
 def scale_shift_act(x, scale, shift, act=None):
     """act(scale[b, c] * x + shift[b, c]) -> bf16, same shape."""
     if not supported(x):

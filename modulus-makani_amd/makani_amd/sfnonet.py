@@ -129,8 +129,8 @@ class SpectralFilterLayer(nn.Module):
         self.filter = SpectralConv(forward_transform, inverse_transform, embed_dim, embed_dim, operator_type=operator_type, separable=separable,
                                    bias=bias, gain=gain)
 
-    def forward(self, x):
-        return self.filter(x)
+    def forward(self, x, lat_stats=False):
+        return self.filter(x, lat_stats=lat_stats) if lat_stats else self.filter(x)
 
 
 class FourierNeuralOperatorBlock(nn.Module):
@@ -186,11 +186,15 @@ class FourierNeuralOperatorBlock(nn.Module):
             return False
         return hasattr(self, "outer_skip") and _is_conv1x1(self.outer_skip) and self.outer_skip.bias is None
 
-    def _forward_fused(self, x, residual):
-        """norm0 -> GELU -> MLP -> norm1 -> + outer_skip(residual) in five kernels: row statistics, scale/shift + GELU,
-        two 1x1 convolutions with bias (+ GELU) epilogues, row statistics, and the skip convolution whose epilogue adds
-        the normalised MLP output."""
-        sc, sh = _norm_coeffs(self.norm0, x)
+    def _forward_fused(self, x, residual, lat_stats=None):
+        """norm0 -> GELU -> MLP -> norm1 -> + outer_skip(residual) in five kernels: row statistics (or, for norm0, the
+        per-latitude moments the inverse transform delivered with x), scale/shift + GELU, two 1x1 convolutions with bias
+        (+ GELU) epilogues, row statistics, and the skip convolution whose epilogue adds the normalised MLP output."""
+        if lat_stats is not None and isinstance(self.norm0, nn.InstanceNorm2d):
+            m = self.norm0
+            sc, sh = pw.instance_norm_coeffs_lat(lat_stats, x.shape[0], m.weight if m.affine else None, m.bias if m.affine else None, m.eps)
+        else:
+            sc, sh = _norm_coeffs(self.norm0, x)
         if sc is None:
             sc = torch.ones(x.shape[:2], dtype=torch.float32, device=x.device)
             sh = torch.zeros_like(sc)
@@ -200,10 +204,15 @@ class FourierNeuralOperatorBlock(nn.Module):
         return pw.conv1x1(residual, self.outer_skip.weight, None, None, x, sc, sh)
 
     def forward(self, x):
-        x, residual = self.filter(x)
+        # on the fused inference path the inverse transform hands over the moments norm0 needs together with its output
+        want_stats = getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and self._fusable()
+        if want_stats:
+            x, residual, lat_stats = self.filter(x, lat_stats=True)
+        else:
+            (x, residual), lat_stats = self.filter(x), None
         if getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 \
                 and residual.shape[2:] == x.shape[2:] and self._fusable():
-            return self._forward_fused(x.contiguous(), residual.contiguous())
+            return self._forward_fused(x.contiguous(), residual.contiguous(), lat_stats)
         x = self.norm0(x)
         if hasattr(self, "inner_skip"):
             x = x + self.inner_skip(residual)

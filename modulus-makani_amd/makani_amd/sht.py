@@ -349,6 +349,23 @@ class InverseRealSHT(_SHTBase):
         out = _SynthesisFn.apply(spec.contiguous(), self, tuple(lead), fused)
         return out if out.dtype == dtype else out.to(dtype)
 
+    def synthesis_with_lat_stats(self, spec, lead, dtype=torch.float32):
+        """synthesis() without autograd that also returns float32 [rows, nlat, 2]: per channel row and latitude the mean
+        over longitude of the field and of its squared deviation from that mean (a by-product of the longitude kernel,
+        enough for the instance norm that follows); (field, None) where the longitude length has no specialised kernel."""
+        rows = _rows(lead)
+        assert tuple(spec.shape) == self.spectral_shape(rows) and spec.dtype == torch.float32
+        plan = self.plan(spec.device)
+        if not lib.sfno_sht_lat_stats_supported(plan.handle):
+            return self.synthesis(spec, lead, dtype), None
+        fused = dtype == torch.bfloat16
+        out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.bfloat16 if fused else torch.float32, device=spec.device)
+        stats = torch.empty((rows, self.nlat, 2), dtype=torch.float32, device=spec.device)
+        ws, nbytes = self.workspace(plan, rows, spec.device)
+        check(lib.sfno_sht_synthesis_lat_stats(plan.handle, _ptr(spec.contiguous()), _ptr(out), _lib.DTYPE_BF16 if fused else _lib.DTYPE_F32, rows,
+                                               _ptr(ws), nbytes, _ptr(stats), _stream_ptr(spec.device)), "sfno_sht_synthesis_lat_stats")
+        return (out if out.dtype == dtype else out.to(dtype)), stats
+
     def _synthesis(self, spec, lead, fused):
         rows = _rows(lead)
         plan = self.plan(spec.device)

@@ -73,10 +73,13 @@ class SpectralConv(nn.Module):
         # coefficients of a spherical transform vanish for l < m; the planar pair fills the whole rectangle
         self._triangular = not getattr(forward_transform, "_planar", False)
 
-    def forward(self, x):
+    def forward(self, x, lat_stats=False):
+        """Returns (x, residual) as the reference does.  With lat_stats=True (inference on the fused path only) a third value
+        follows: per-latitude moments of x from InverseRealSHT.synthesis_with_lat_stats, or None where they are not available."""
         dtype = x.dtype
         residual = x
         B, C, H, W = x.shape
+        stats = None
 
         if self._fused:
             # The transforms and the contraction work in float32 regardless of autocast.  A bf16 input is
@@ -87,7 +90,10 @@ class SpectralConv(nn.Module):
             if self.scale_residual:
                 residual = self.inverse_transform.synthesis(spec, (B, C), dtype=dtype if dtype == torch.bfloat16 else torch.float32).to(dtype)
             spec = dhconv_spectral(spec, self.weight, B, self.modes_lon, triangular=self._triangular, compute=self.compute)
-            x = self.inverse_transform.synthesis(spec, (B, self.out_channels), dtype=dtype if fuse_cast else torch.float32)
+            if lat_stats and fuse_cast and not torch.is_grad_enabled():
+                x, stats = self.inverse_transform.synthesis_with_lat_stats(spec, (B, self.out_channels), dtype=dtype)
+            else:
+                x = self.inverse_transform.synthesis(spec, (B, self.out_channels), dtype=dtype if fuse_cast else torch.float32)
         else:
             x = x.float()
             with torch.autocast(device_type="cuda", enabled=False):
@@ -103,4 +109,4 @@ class SpectralConv(nn.Module):
         if hasattr(self, "bias"):
             x = x + self.bias
         x = x.to(dtype=dtype)
-        return x, residual
+        return (x, residual, stats) if lat_stats else (x, residual)

@@ -114,3 +114,48 @@ def test_unsupported_inputs_raise(lib_built):
         pw.conv1x1(torch.randn(1, 4, 3, 5).bfloat16().cuda(), w)      # H*W not a multiple of 8
     with pytest.raises(RuntimeError):
         pw.conv1x1(torch.randn(1, 4, 4, 8).bfloat16(), w.cpu())       # CPU tensor
+
+
+@pytest.mark.parametrize("nlat,nlon,lmax,mmax,lead,dtype", [
+    (24, 64, 24, 33, (2, 5), torch.float32),          # Nyquist order kept; odd channel count (one padded slot in the last pair)
+    (31, 480, 31, 40, (1, 9), torch.bfloat16),
+    (40, 180, 30, 31, (3, 4), torch.bfloat16),
+])
+def test_instance_norm_coeffs_from_latitude_moments(lib_built, nlat, nlon, lmax, mmax, lead, dtype):
+    """The inverse transform's by-product (per-latitude mean and mean squared deviation over longitude, by Parseval on the
+    Fourier coefficients) gives the instance-norm statistics of the field it writes: (scale, shift) against float64
+    statistics of the float32 field, and the field itself unchanged."""
+    import makani_amd as ma
+    from makani_amd import pointwise as pw
+
+    print(f"case lat-moments {nlat}x{nlon} l{lmax} m{mmax} lead={lead} {dtype}", flush=True)
+    torch.manual_seed(31)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid="legendre-gauss")
+    B, C = lead
+    c = torch.randn(B, C, lmax, mmax, dtype=torch.complex64) * torch.exp(torch.randn(B, C, 1, 1))
+    c[:, :, 0, 0] += 3.0 * torch.randn(B, C)                     # channel means well away from zero
+    spec = torch.zeros(isht.spectral_shape(B * C), device="cuda")
+    from makani_amd._lib import lib, check
+    import ctypes
+    check(lib.sfno_coeffs_to_spectral(ctypes.c_void_p(c.cuda().contiguous().data_ptr()), ctypes.c_void_p(spec.data_ptr()), B * C, lmax, mmax, 1,
+                                      ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "to_spectral")
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        x32 = isht.synthesis(spec, (B, C))
+        x, stats = isht.synthesis_with_lat_stats(spec, (B, C), dtype=dtype)
+    assert stats is not None and tuple(stats.shape) == (B * C, nlat, 2)
+    assert torch.equal(x, x32.to(dtype))
+    gamma, beta = torch.randn(C).cuda(), torch.randn(C).cuda()
+    sc, sh = pw.instance_norm_coeffs_lat(stats, B, gamma, beta, 1e-6)
+    torch.cuda.synchronize()
+    xd = x32.double().cpu()
+    mean, var = xd.mean(dim=(2, 3)), xd.var(dim=(2, 3), unbiased=False)
+    want_sc = gamma.cpu().double()[None, :] / torch.sqrt(var + 1e-6)
+    want_sh = beta.cpu().double()[None, :] - mean * want_sc
+    assert rel_l2(sc, want_sc) < 1e-5
+    assert rel_l2(sh, want_sh) < 1e-5
+    # per-latitude values themselves
+    a = xd.mean(dim=3).reshape(B * C, nlat)
+    d = ((xd - xd.mean(dim=3, keepdim=True)) ** 2).mean(dim=3).reshape(B * C, nlat)
+    assert rel_l2(stats[..., 0], a) < 1e-5
+    assert rel_l2(stats[..., 1], d) < 1e-5

@@ -103,6 +103,34 @@ def test_torch_restatement_matches_numpy_oracle(nlat, nlon, lmax, mmax):
     assert np.abs(ref.inverse(torch.from_numpy(c)).numpy() - fft2_inverse(c, t)).max() < 1e-12
 
 
+def _golden():
+    import os
+
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", "fft2_24x32_known_answers.npz"))
+
+
+def test_oracle_against_committed_known_answers():
+    """tests/golden/fft2_24x32_known_answers.npz holds the defining double sums (made by tests/golden/make_golden_fft2.py
+    without any FFT routine): the oracle reproduces them."""
+    g = _golden()
+    t = Fft2Modes(int(g["nlat"]), int(g["nlon"]), int(g["lmax"]), int(g["mmax"]))
+    assert np.abs(fft2_forward(g["x"].astype(np.float64), t) - g["forward"]).max() < 1e-12
+    assert np.abs(fft2_inverse(g["coeffs"].astype(np.complex128), t) - g["inverse"]).max() < 1e-12
+
+
+@pytest.mark.gpu
+def test_hip_path_against_committed_known_answers(lib_built):
+    import makani_amd as ma
+
+    g = _golden()
+    nlat, nlon, lmax, mmax = int(g["nlat"]), int(g["nlon"]), int(g["lmax"]), int(g["mmax"])
+    y = ma.RealFFT2(nlat, nlon, lmax, mmax)(torch.from_numpy(g["x"]).cuda())
+    z = ma.InverseRealFFT2(nlat, nlon, lmax, mmax)(torch.from_numpy(g["coeffs"]).cuda())
+    torch.cuda.synchronize()
+    assert rel_l2(y.cpu().numpy(), g["forward"]) < TOL
+    assert rel_l2(z.cpu().numpy(), g["inverse"]) < TOL
+
+
 def test_modules_mirror_the_reference_attributes():
     import makani_amd as ma
 

@@ -159,3 +159,26 @@ def test_instance_norm_coeffs_from_latitude_moments(lib_built, nlat, nlon, lmax,
     d = ((xd - xd.mean(dim=3, keepdim=True)) ** 2).mean(dim=3).reshape(B * C, nlat)
     assert rel_l2(stats[..., 0], a) < 1e-5
     assert rel_l2(stats[..., 1], d) < 1e-5
+
+
+def test_latitude_moments_absent_without_specialised_longitude_kernel(lib_built):
+    """A longitude length served by the run-time radix kernels delivers no moments: the caller gets None and falls back to
+    the statistics pass; the C entry point says unsupported."""
+    import ctypes
+
+    import makani_amd as ma
+    from makani_amd._lib import lib
+
+    isht = ma.InverseRealSHT(12, 50, lmax=12, mmax=13, grid="legendre-gauss")
+    spec = torch.zeros(isht.spectral_shape(4), device="cuda")
+    with torch.no_grad():
+        x, stats = isht.synthesis_with_lat_stats(spec, (1, 4))
+    assert stats is None and tuple(x.shape) == (1, 4, 12, 50)
+    plan = isht.plan(spec.device)
+    assert lib.sfno_sht_lat_stats_supported(plan.handle) == 0
+    ws, nbytes = isht.workspace(plan, 4, spec.device)
+    out = torch.empty(1, 4, 12, 50, device="cuda")
+    st = torch.empty(4, 12, 2, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.sfno_sht_synthesis_lat_stats(plan.handle, P(spec), P(out), 0, 4, P(ws), nbytes, P(st), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == -5

@@ -57,16 +57,21 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
     // [buffer][parity][k][column]; reused for the parity exchange of the synthesis epilogue
     __shared__ __align__(16) float qs[2][2][PG_KC][LDQ];
 
-    const int2 wi = a.work[blockIdx.x];
+    // Workgroups go to the 8 XCDs round-robin by linear id and entry 8 i + x of the work list is meant for XCD x: the
+    // column tiles of one entry run back to back on that XCD, where they share the entry's table fragments in L2.
+    const int nct = (a.ld + 32 * NT - 1) / (32 * NT);
+    const int qid = blockIdx.x >> 3;
+    const int ct = qid % nct;
+    const int2 wi = a.work[(qid / nct) * 8 + (blockIdx.x & 7)];
     const int m = wi.x;
     if (m < 0) return;
     // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     // wavefront w runs on SIMD w; alternate which SIMDs get the (possibly absent) second row block
     // and the (one row shorter) odd parity from workgroup to workgroup
-    const int wslot = (wave + blockIdx.x) & 3;
+    const int wslot = (wave + qid) & 3;
     const int par = wslot >> 1, rb = wi.y + (wslot & 1);
-    const int n0 = blockIdx.y * TN;
+    const int n0 = ct * TN;
     const int ld = a.ld, nlat = a.nlat, lmax = a.lmax;
     if (n0 >= ld) return;
     const int K2 = (nlat + 1) >> 1;
@@ -297,7 +302,9 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
     }
 #define LF_CASE(NT_)                                                                                 \
     case NT_: {                                                                                      \
-        dim3 grid(n_work, (unsigned)((ncols + 32 * NT_ - 1) / (32 * NT_)));                          \
+        const int64_t nwg = (int64_t)n_work * ((ncols + 32 * NT_ - 1) / (32 * NT_));                 \
+        if (nwg > 0x7fffffffLL) return SFNO_EUNSUPPORTED;                                            \
+        dim3 grid((unsigned)nwg);                                                                    \
         hipLaunchKernelGGL((legendre_fold_kernel<NT_, ANALYSIS, MODE>), grid, dim3(256), 0, s, a);   \
         break;                                                                                       \
     }

@@ -244,3 +244,34 @@ def test_every_specialised_longitude_length(lib_built, nlon):
     m, l = torch.arange(mmax)[:, None], torch.arange(nlat)[None, :]
     keep = (m <= l).cuda()
     assert torch.equal(a[..., : 2 * 10][keep], b[..., : 2 * 10][keep])
+
+
+def test_empty_ragged_and_strided_inputs(lib_built):
+    """Edge shapes at the module boundary: no leading dimensions, an empty batch, a non-contiguous view, half and double
+    precision inputs (the reference up-casts half inputs itself; float64 is not this path's arithmetic)."""
+    import makani_amd as ma
+
+    nlat, nlon = 12, 24
+    sht, isht = ma.RealSHT(nlat, nlon, grid="legendre-gauss"), ma.InverseRealSHT(nlat, nlon, grid="legendre-gauss")
+    fft, ifft = ma.RealFFT2(nlat, nlon), ma.InverseRealFFT2(nlat, nlon)
+    t = ShtTables(nlat, nlon, None, None, "legendre-gauss")
+    torch.manual_seed(12)
+    x = torch.randn(nlat, nlon)
+    for f, inv in ((sht, isht), (fft, ifft)):
+        y = f(x.cuda())                                         # a single field, no batch or channel axis
+        assert tuple(y.shape) == (f.lmax, f.mmax)
+        assert tuple(inv(y).shape) == (nlat, nlon)
+        e = f(torch.empty(0, 3, nlat, nlon, device="cuda"))      # empty batch
+        assert tuple(e.shape) == (0, 3, f.lmax, f.mmax)
+        assert tuple(inv(e).shape) == (0, 3, nlat, nlon)
+    assert rel_l2(sht(x.cuda()).cpu().numpy(), sht_forward(x.double().numpy(), t)) < TOL
+    big = torch.randn(2, nlat, 3, nlon)
+    view = big.permute(0, 2, 1, 3)                               # [2, 3, nlat, nlon], not contiguous
+    got = sht(view.cuda())
+    assert rel_l2(got.cpu().numpy(), sht_forward(view.double().numpy(), t)) < TOL
+    half = torch.randn(2, nlat, nlon).half()
+    assert rel_l2(sht(half.cuda()).cpu().numpy(), sht_forward(half.double().numpy(), t)) < TOL
+    with pytest.raises(TypeError):
+        sht(torch.randn(2, nlat, nlon, dtype=torch.float64).cuda())
+    with pytest.raises(TypeError):
+        isht(torch.randn(2, isht.lmax, isht.mmax).cuda())        # real input where coefficients are expected

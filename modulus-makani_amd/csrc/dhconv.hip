@@ -27,27 +27,61 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f2 __attribute__((ext_vector_type(2)));
 
-// grid = (8 * ceil(L/8) * nob, row groups); VEC4: 2*I is a multiple of 4 so activation rows can be read as float4
+// Workgroup -> (degree, column block, row group).  Workgroups go to the 8 XCDs round-robin by linear id.  All column
+// blocks and row groups of a degree share its activation panel, and the row groups of one (degree, column block) share
+// its weights, so a degree stays on one XCD and its workgroups are neighbours in that XCD's queue, row groups fastest.
+// Only row groups that exist are enumerated (a degree has (l + 1) B rows): XCD x serves the degrees L-1-x, L-9-x, ...
+// (largest first: they have the most orders, hence the most rows) and a workgroup finds its place by walking that list.
+__device__ __forceinline__ bool dh_map(const DhconvArgs& a, int group, int& l, int& ob, int& r0, int& ncols, int& rot) {
+    int q = blockIdx.x >> 3;
+    for (int lidx = blockIdx.x & 7; lidx < a.L; lidx += 8) {
+        const int ll = a.L - 1 - lidx;
+        const int nc_l = (a.tri ? min(ll + 1, a.M) : a.M) * a.B;      // rows (m, b) present at this degree
+        const int t = (nc_l + group - 1) / group;
+        const int n = a.nob * t;
+        if (q < n) {
+            l = ll;
+            ob = q / t;
+            const int rt = q - ob * t;
+            r0 = rt * group;
+            ncols = nc_l;
+            rot = lidx + ob + rt;
+            return true;
+        }
+        q -= n;
+    }
+    return false;
+}
+
+// number of workgroups dh_map enumerates: 8 x the longest XCD queue
+static int64_t dh_blocks(const DhconvArgs& a, int group) {
+    int64_t longest = 0;
+    for (int x = 0; x < 8; ++x) {
+        int64_t n = 0;
+        for (int lidx = x; lidx < a.L; lidx += 8) {
+            const int ll = a.L - 1 - lidx;
+            const int64_t nc_l = (int64_t)(a.tri ? (ll + 1 < a.M ? ll + 1 : a.M) : a.M) * a.B;
+            n += a.nob * ((nc_l + group - 1) / group);
+        }
+        longest = n > longest ? n : longest;
+    }
+    return 8 * longest;
+}
+
+
+// grid = dh_blocks workgroups (see dh_map), row groups of DH_GROUP; VEC4: 2*I is a multiple of 4 so activation rows can be read as float4
 constexpr int DH_GROUP = 64;                         // rows (m,b) per workgroup
 template <bool VEC4>
 __global__ __launch_bounds__(256, 4) void dhconv_kernel(DhconvArgs a) {
     constexpr int LDW = DH_COLS / 2 + 32;            // plane pitch = 32 mod 64: the two half-waves read different banks
     __shared__ __align__(16) float ws[2][3][8][LDW]; // [buffer][plane][input channel of the chunk][output channel]
 
-    // Workgroups go to the 8 XCDs round-robin by linear id: all column blocks and row groups of a
-    // degree share their activation panel, so a degree stays on one XCD.  Degrees are handed out
-    // largest first: they have the most orders, hence the most rows.
-    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-    const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
-    if (lidx >= a.L) return;
-    const int l = a.L - 1 - lidx;
+    int l, ob, r0, ncols, rot;
+    if (!dh_map(a, DH_GROUP, l, ob, r0, ncols, rot)) return;
     // Wavefront w of every workgroup runs on SIMD w, and low degrees fill only the first row blocks:
     // rotate the block a wavefront takes from workgroup to workgroup so that no SIMD gets all the work.
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
-    const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;      // rows (m,b) present at this degree
-    const int r0 = blockIdx.y * DH_GROUP;
-    if (r0 >= ncols) return;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + rot) & 3;
     // wavefront = (row block of 32, column tile of 32 output channels)
     const int nrb = min(DH_GROUP / 32, (ncols - r0 + 31) / 32);
     const int rb = wave >> 1, t0 = wave & 1;
@@ -199,21 +233,16 @@ __device__ __forceinline__ bf16x8 to_bf16x8(f4 a, f4 b) {
     return v;
 }
 
-// grid = (8 * ceil(L/8) * nob, row groups of 128), nob = ceil(2*O / 256); requires 2*I % 8 == 0
+// grid = dh_blocks workgroups (see dh_map), row groups of 128, nob = ceil(2*O / 256); requires 2*I % 8 == 0
 __global__ __launch_bounds__(256, 2) void dhconv_bf16_kernel(DhconvArgs a) {
     constexpr int NT = DHB_COLS / 32;                // 8 column tiles per wavefront
     constexpr int PITCH = DHB_KC + 8;                // bf16 elements per LDS row (80 bytes: 16-byte reads of 16 lanes hit distinct banks)
     __shared__ __align__(16) unsigned short ws[2][DHB_COLS][PITCH];
 
-    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-    const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
-    if (lidx >= a.L) return;
-    const int l = a.L - 1 - lidx;
+    int l, ob, r0, ncols, rot;
+    if (!dh_map(a, 128, l, ob, r0, ncols, rot)) return;
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
-    const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;
-    const int r0 = blockIdx.y * 128;
-    if (r0 >= ncols) return;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + rot) & 3;
     const bool active = r0 + 32 * wave < ncols;
     const int nc = a.nc;                                           // chunks of 32 i'
     const int kg = lane >> 5, cl = lane & 31;
@@ -342,8 +371,9 @@ int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s) {
     const int64_t rows_max = (int64_t)a.M * a.B;
     if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
     if (a.I2 % 4 != 0 || a.ld_in % 4 != 0) return SFNO_EUNSUPPORTED;
-    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
-    hipLaunchKernelGGL(dhconv_bf16_kernel, grid, dim3(256), 0, s, a);
+    const int64_t blocks = dh_blocks(a, 128);
+    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
@@ -374,22 +404,17 @@ __device__ __forceinline__ void dh_split3(float a, float b, unsigned int& hi, un
 // its SIMD), so the kernel is software-pipelined by hand: while the 24 matrix instructions of chunk c are issued, the
 // activations of chunk c+1 are split and the weights of chunk c+1 are expanded into the other LDS buffer, a few vector
 // instructions after each matrix instruction, behind scheduling fences; the loads run two chunks ahead.
-// grid = (8 * ceil(L/8) * nob, row groups of 128), nob = ceil(2*O / 128); requires 2*I % 4 == 0
+// grid = dh_blocks workgroups (see dh_map), row groups of 128, nob = ceil(2*O / 128); requires 2*I % 4 == 0
 __global__ __launch_bounds__(256, 3) void dhconv_split_kernel(DhconvArgs a) {
     constexpr int NT = DHS_COLS / 32;                // 4 column tiles per wavefront
     constexpr int PITCH = DHS_KC + 8;                // bf16 elements per LDS row (48 bytes: 16-byte reads of 8 lanes hit distinct banks)
     constexpr int PLANE = DHS_COLS * PITCH;
     __shared__ __align__(16) unsigned short ws[2][3][DHS_COLS][PITCH];
 
-    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-    const int lidx = (q / a.nob) * 8 + xcd, ob = q % a.nob;
-    if (lidx >= a.L) return;
-    const int l = a.L - 1 - lidx;
+    int l, ob, r0, ncols, rot;
+    if (!dh_map(a, 128, l, ob, r0, ncols, rot)) return;
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + q + blockIdx.y) & 3;
-    const int ncols = (a.tri ? min(l + 1, a.M) : a.M) * a.B;
-    const int r0 = blockIdx.y * 128;
-    if (r0 >= ncols) return;
+    const int wave = (__builtin_amdgcn_readfirstlane(tid >> 6) + rot) & 3;
     const bool active = r0 + 32 * wave < ncols;
     const int nc = a.nc;                                           // chunks of 16 i'
     const int kg = lane >> 5, cl = lane & 31;
@@ -599,15 +624,18 @@ int dhconv_split_launch(const DhconvArgs& a, hipStream_t s) {
     const int64_t rows_max = (int64_t)a.M * a.B;
     if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
     if (a.I2 % 4 != 0 || a.ld_in % 4 != 0) return SFNO_EUNSUPPORTED;
-    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + 127) / 128));
-    hipLaunchKernelGGL(dhconv_split_kernel, grid, dim3(256), 0, s, a);
+    const int64_t blocks = dh_blocks(a, 128);
+    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_split_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 
 int dhconv_launch(const DhconvArgs& a, hipStream_t s) {
     const int64_t rows_max = (int64_t)a.M * a.B;
     if (rows_max <= 0 || a.L <= 0) return SFNO_OK;
-    dim3 grid((unsigned)((a.L + 7) / 8 * 8 * a.nob), (unsigned)((rows_max + DH_GROUP - 1) / DH_GROUP));
+    const int64_t blocks = dh_blocks(a, DH_GROUP);
+    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    const dim3 grid((unsigned)blocks);
     const bool vec4 = a.I2 % 4 == 0 && a.ld_in % 4 == 0;
     if (vec4)
         hipLaunchKernelGGL((dhconv_kernel<true>), grid, dim3(256), 0, s, a);

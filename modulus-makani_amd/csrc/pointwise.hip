@@ -572,10 +572,10 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
 }
 
 int row_stats_segments(int64_t rows, int64_t P) {
-    // enough workgroups to fill the chip, at least ~16 K elements each
-    int64_t nseg = (2048 + rows - 1) / rows;
-    nseg = std::min<int64_t>(nseg, std::max<int64_t>(1, P / 16384));
-    return (int)std::max<int64_t>(1, std::min<int64_t>(nseg, 64));
+    // ~16 K elements per workgroup.  The split depends on the row length only, so that the sums of a row (and with them
+    // every value downstream) do not change with the number of rows: a sample gives the same result alone and in a batch.
+    (void)rows;
+    return (int)std::max<int64_t>(1, std::min<int64_t>(P / 16384, 64));
 }
 
 int instance_norm_coeffs_launch(const unsigned short* x, const float* gamma, const float* beta, float* scale, float* shift, float2* partial,

@@ -36,40 +36,51 @@ class SfnoOracle:
 
     @staticmethod
     def _conv(x, sd, name):
-        w = sd[name + ".weight"].double()
+        w = sd[name + ".weight"].double().to(x.device)
         b = sd.get(name + ".bias")
+        if x.is_cuda:
+            # a 1x1 convolution is a matrix product over channels; float64 convolutions have no device library behind them
+            y = torch.einsum("oi,bihw->bohw", w[:, :, 0, 0], x)
+            return y if b is None else y + b.double().to(x.device)[None, :, None, None]
         return F.conv2d(x, w, None if b is None else b.double())
 
     def _norm(self, x, sd, name):
         if self.normalization == "none":
             return x
-        return F.instance_norm(x, weight=sd[name + ".weight"].double(), bias=sd[name + ".bias"].double(), eps=1e-6)
+        return F.instance_norm(x, weight=sd[name + ".weight"].double().to(x.device), bias=sd[name + ".bias"].double().to(x.device), eps=1e-6)
 
-    def forward(self, sd, x):
+    def forward(self, sd, x, pointwise_device="cpu", taps=None):
+        """pointwise_device: where the float64 torch ops between the spectral operators run ("cpu", or a HIP device for the
+        full-size model, whose 1x1 convolutions are 4.5 TFLOP per sample); the spectral operators always run on the numpy
+        oracle.  taps: optional dict that receives the input of every SpectralConv (key = block index) as a CPU tensor."""
         sd = {k: v.detach().cpu() for k, v in sd.items()}
+        dev = torch.device(pointwise_device)
         x = x.detach().cpu().double()
         if self.big_skip:
             if self.out_shape != self.inp_shape:
                 residual = torch.from_numpy(transform_inverse(transform_forward(x.numpy(), self.down), self.up))
             else:
                 residual = x
-        y = self._conv(self.act(self._conv(x, sd, "encoder.fwd.0")), sd, "encoder.fwd.2")
+        residual = residual.to(dev) if self.big_skip else None
+        y = self._conv(self.act(self._conv(x.to(dev), sd, "encoder.fwd.0")), sd, "encoder.fwd.2")
         # position embedding (sfnonet.py:612-622): a learnt field, or learnt coefficients synthesised on the input grid
         if "pos_embed" in sd:
-            y = y + sd["pos_embed"].double()
+            y = y + sd["pos_embed"].double().to(dev)
         elif "pos_embed.0" in sd:
             re, im = sd["pos_embed.0"].double().numpy(), sd["pos_embed.1"].double().numpy()
             c = re + 1j * np.pad(im, ((0, 0), (0, 0), (0, 0), (1, 0)))
-            y = y + torch.from_numpy(transform_inverse(c, self.up))
+            y = y + torch.from_numpy(transform_inverse(c, self.up)).to(dev)
         for i in range(self.num_layers):
             fwd = self.down if i == 0 else self.mid
             inv = self.up if i == self.num_layers - 1 else self.mid
             p = f"blocks.{i}."
             w = sd[p + "filter.filter.weight"].numpy().astype(np.complex128)
-            z, res = spectral_conv(y.numpy(), w, fwd, inv)
-            z, res = torch.from_numpy(z), torch.from_numpy(np.asarray(res))
+            if taps is not None:
+                taps[i] = y.cpu()
+            z, res = spectral_conv(y.cpu().numpy(), w, fwd, inv)
+            z, res = torch.from_numpy(z).to(dev), torch.from_numpy(np.asarray(res)).to(dev)
             if p + "filter.filter.bias" in sd:           # spectral_convolution.py:143-144
-                z = z + sd[p + "filter.filter.bias"].double()
+                z = z + sd[p + "filter.filter.bias"].double().to(dev)
             z = self.act(self._norm(z, sd, p + "norm0"))
             if self.use_mlp:
                 z = self._conv(self.act(self._conv(z, sd, p + "mlp.fwd.0")), sd, p + "mlp.fwd.3")
@@ -78,4 +89,4 @@ class SfnoOracle:
         y = self._conv(self.act(self._conv(y, sd, "decoder.fwd.0")), sd, "decoder.fwd.2")
         if self.big_skip:
             y = y + self._conv(residual, sd, "residual_transform")
-        return y
+        return y.cpu()

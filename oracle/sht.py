@@ -12,6 +12,7 @@ makani/models/networks/sfnonet.py:596,598,616):
             Nyquist bins is dropped, bins >= mmax are zero)
 """
 import numpy as np
+import scipy.fft
 
 from .quadrature import grid_nodes, default_lmax
 from .legendre import legpoly
@@ -61,13 +62,14 @@ class ShtTables:
 
 def rfft_lon(x, mmax):
     """Longitude stage of the forward transform: 2 pi/nlon * sum_n x e^{-i m phi_n}, m < mmax."""
-    X = 2.0 * np.pi * np.fft.rfft(x, axis=-1, norm="forward")
+    # scipy.fft is numpy's FFT routine with a thread pool (the full-resolution checks transform 384 x 721 rows)
+    X = 2.0 * np.pi * scipy.fft.rfft(x, axis=-1, norm="forward", workers=-1)
     return X[..., :mmax]
 
 
 def irfft_lon(X, nlon):
     """Longitude stage of the inverse: unnormalised C2R inverse DFT, zero-padded to nlon//2+1."""
-    return np.fft.irfft(X, n=nlon, axis=-1, norm="forward")
+    return scipy.fft.irfft(X, n=nlon, axis=-1, norm="forward", workers=-1)
 
 
 def legendre_analysis(X, weights):
@@ -80,12 +82,16 @@ def legendre_analysis(X, weights):
     lead = X.shape[:-2]
     Xf = np.ascontiguousarray(X).reshape(-1, nlat, X.shape[-1])
     rows = Xf.shape[0]
-    c = np.zeros((rows, lmax, mmax), dtype=np.complex128)
+    # order-major copies, so that every per-order product reads and writes contiguous memory
+    # (real and imaginary planes apart: the strided .real / .imag views of a complex array would take numpy's own loop
+    # instead of the BLAS routine)
+    Xr = np.ascontiguousarray(Xf.real.transpose(2, 0, 1))  # (mmax, rows, nlat)
+    Xi = np.ascontiguousarray(Xf.imag.transpose(2, 0, 1))
+    ct = np.zeros((mmax, rows, lmax), dtype=np.complex128)
     for m in range(min(mmax, lmax)):
-        xm = np.ascontiguousarray(Xf[:, :, m])             # (rows, nlat) complex
-        w = np.ascontiguousarray(weights[m, m:, :])        # (lmax-m, nlat) real
-        c[:, m:, m] = (xm.real @ w.T) + 1j * (xm.imag @ w.T)
-    return c.reshape(*lead, lmax, mmax)
+        w = np.ascontiguousarray(weights[m, m:, :].T)      # (nlat, lmax-m) real
+        ct[m, :, m:] = (Xr[m] @ w) + 1j * (Xi[m] @ w)
+    return np.ascontiguousarray(ct.transpose(1, 2, 0)).reshape(*lead, lmax, mmax)
 
 
 def legendre_synthesis(c, pct):
@@ -94,19 +100,20 @@ def legendre_synthesis(c, pct):
     lead = c.shape[:-2]
     cf = np.ascontiguousarray(c).reshape(-1, lmax, mmax)
     rows = cf.shape[0]
-    X = np.zeros((rows, nlat, mmax), dtype=np.complex128)
+    cr = np.ascontiguousarray(cf.real.transpose(2, 0, 1))  # (mmax, rows, lmax)
+    ci = np.ascontiguousarray(cf.imag.transpose(2, 0, 1))
+    Xt = np.zeros((mmax, rows, nlat), dtype=np.complex128)
     for m in range(min(mmax, lmax)):
-        cm = np.ascontiguousarray(cf[:, m:, m])            # (rows, lmax-m)
         p = np.ascontiguousarray(pct[m, m:, :])            # (lmax-m, nlat)
-        X[:, :, m] = (cm.real @ p) + 1j * (cm.imag @ p)
-    return X.reshape(*lead, nlat, mmax)
+        Xt[m] = (np.ascontiguousarray(cr[m, :, m:]) @ p) + 1j * (np.ascontiguousarray(ci[m, :, m:]) @ p)
+    return np.ascontiguousarray(Xt.transpose(1, 2, 0)).reshape(*lead, nlat, mmax)
 
 
 def sht_forward(x, tables):
     x = np.asarray(x)
     assert x.shape[-2] == tables.nlat
     assert x.shape[-1] == tables.nlon
-    X = rfft_lon(x.astype(np.float64), tables.mmax)
+    X = rfft_lon(np.asarray(x, dtype=np.float64), tables.mmax)
     # weights[m, l, k] = P[m, l, k] * w[k]: fold w into X instead of materialising a second table
     return legendre_analysis(X * tables.quad_w[:, None], tables.p_analysis)
 
@@ -115,5 +122,5 @@ def sht_inverse(c, tables):
     c = np.asarray(c)
     assert c.shape[-2] == tables.lmax
     assert c.shape[-1] == tables.mmax
-    X = legendre_synthesis(c.astype(np.complex128), tables.pct)
+    X = legendre_synthesis(np.asarray(c, dtype=np.complex128), tables.pct)
     return irfft_lon(X, tables.nlon)

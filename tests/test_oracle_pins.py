@@ -253,6 +253,23 @@ def test_dhconv_brute_force():
     assert np.allclose(dhconv(x[:, :, :1], w[:, :, :1])[:, :, 0], np.einsum("bim,io->bom", x[:, :, 0], w[:, :, 0]))
 
 
+def test_dhconv_many_channels_brute_force():
+    """From 64 x 64 channels on the oracle evaluates the sum as matrix products; same brute-force loop pins that branch
+    (distinct extents everywhere, so a transposed operand cannot pass)."""
+    rng = np.random.default_rng(11)
+    B, I, O, L, M = 2, 70, 64, 2, 3
+    x = rng.standard_normal((B, I, L, M)) + 1j * rng.standard_normal((B, I, L, M))
+    w = rng.standard_normal((I, O, L)) + 1j * rng.standard_normal((I, O, L))
+    y = np.zeros((B, O, L, M), dtype=complex)
+    for b in range(B):
+        for o in range(O):
+            for l in range(L):
+                for m in range(M):
+                    y[b, o, l, m] = sum(x[b, i, l, m] * w[i, o, l] for i in range(I))
+    got = dhconv(x, w)
+    assert got.shape == y.shape and np.allclose(got, y, atol=1e-12)
+
+
 def test_diagonal_brute_force():
     from oracle.dhconv import diagonal
 

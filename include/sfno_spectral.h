@@ -139,6 +139,17 @@ int sfno_sht_forward(const sfno_sht_plan* plan, const float* x, void* coeffs, in
 int sfno_sht_inverse(const sfno_sht_plan* plan, const void* coeffs, float* x, int64_t rows,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* sfno_sht_forward without a workspace argument and without any allocation, for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (PyTorch allocates the intermediates of RealSHT.forward on every call).  The Fourier and spectral-layout
+ * buffers live in one array of SFNO_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process
+ * ends; sfno_sht_plan_create looks up its address for the plan's device.  Returns SFNO_EWORKSPACE when
+ * sfno_sht_workspace_bytes(plan, rows) exceeds the array (64 MiB: e.g. 8 rows of 721 x 1440 with lmax = mmax = 721, or
+ * 64 rows of 241 x 480), SFNO_EHIP when the look-up failed.  Results equal sfno_sht_forward's bit for bit.  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU (different streams or threads) race. */
+#define SFNO_STATIC_SCRATCH_BYTES (64u << 20)
+int sfno_sht_forward_static(const sfno_sht_plan* plan, const float* x, void* coeffs, int64_t rows, void* stream);
+
 /* Same transforms with coefficients kept in the spectral layout (no layout pass).  The grid-side
  * tensor x may be float32 or bfloat16 (`x_dtype`, SFNO_DTYPE_*): a bf16 field is widened on load /
  * rounded to nearest even on store inside the FFT kernels, which is what the reference's

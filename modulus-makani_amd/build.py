@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "makani_amd", "libsfno_spectral.so")
-SOURCES = ["tables.cpp", "capi.cpp", "dhconv.hip", "dhconv_wgrad.hip", "pointwise.hip", "diagonal.hip", "degree_power.hip", "legendre_fold.hip", "fft.hip", "fft_fast.hip", "layout.hip"]
+SOURCES = ["tables.cpp", "capi.cpp", "dhconv.hip", "dhconv_wgrad.hip", "pointwise.hip", "diagonal.hip", "degree_power.hip", "legendre_fold.hip", "fft.hip", "fft_fast.hip", "layout.hip", "static_scratch.hip"]
 HEADERS = [os.path.join(CSRC, "sfno_internal.h"), os.path.join(ROOT, "include", "sfno_spectral.h")]
 
 

@@ -180,6 +180,8 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     p->compute = compute == SFNO_COMPUTE_BF16 ? SFNO_COMPUTE_BF16 : SFNO_COMPUTE_FP32;
     p->format = compute == SFNO_COMPUTE_BF16 ? PG_FORMAT_BF16 : compute == SFNO_COMPUTE_FP32_MFMA ? PG_FORMAT_FP32 : PG_FORMAT_SPLIT;
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return SFNO_EHIP; }
+    // set-up of sfno_sht_forward_static on this device; a failure is reported by that entry point, not here
+    (void)static_scratch_prepare();
     if (grid == SFNO_GRID_PLANAR) {
         int rc = planar_init(p);
         if (rc != SFNO_OK) { sfno_sht_plan_destroy(p); return rc; }

@@ -160,6 +160,10 @@ int latfft_launch(const FftPlan& p, bool inverse, const float* in, float* out, i
 int degree_power_launch(const float* spec, float* power, int64_t rows, int lmax, int mmax, int ld, hipStream_t s);
 int degree_power_grad_launch(const float* spec, const float* gpower, float* gspec, int64_t rows, int lmax, int mmax, int ld, hipStream_t s);
 
+// ---- file-scope scratch array of sfno_sht_forward_static (static_scratch.hip) ----------------
+// looks up, once per device, the device address of the array on the current device; called at plan creation
+int static_scratch_prepare();
+
 // ---- layout passes (layout.hip) ----------------------------------------------------------
 int coeffs_to_spectral_launch(const float2* coeffs, float* spec, int64_t rows, int lmax, int mmax, int ld, int tri,
                               hipStream_t s);

@@ -44,6 +44,7 @@ def _load():
         "sfno_sht_workspace_bytes": (sz, [vp, i64]),
         "sfno_sht_forward": (i32, [vp, vp, vp, i64, vp, sz, vp]),
         "sfno_sht_inverse": (i32, [vp, vp, vp, i64, vp, sz, vp]),
+        "sfno_sht_forward_static": (i32, [vp, vp, vp, i64, vp]),
         "sfno_sht_io_dtype_supported": (i32, [vp, i32]),
         "sfno_sht_analysis": (i32, [vp, vp, i32, vp, i64, vp, sz, vp]),
         "sfno_sht_synthesis": (i32, [vp, vp, vp, i32, i64, vp, sz, vp]),

@@ -237,6 +237,13 @@ int fft_plan_init(FftPlan& p, int n) {
     if (n < 1) return SFNO_EINVAL;
     p.n = n;
     p.npass = 0;
+    {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+            p.n_cu = cus;
+        else
+            (void)hipGetLastError();
+    }
     int rem = n;
     while (rem % 4 == 0) { p.radix[p.npass++] = 4; rem /= 4; }
     while (rem % 2 == 0) { p.radix[p.npass++] = 2; rem /= 2; }
@@ -264,7 +271,9 @@ void fft_plan_free(FftPlan& p) {
     if (p.d_tw1) (void)hipFree(p.d_tw1);
     if (p.d_chirp) (void)hipFree(p.d_chirp);
     if (p.d_vhat) (void)hipFree(p.d_vhat);
+    if (p.d_post) (void)hipFree(p.d_post);
     p.d_tw = p.d_tw0 = p.d_tw1 = p.d_chirp = p.d_vhat = nullptr;
+    p.d_post = nullptr;
     p.chirp_m = 0;
 }
 

@@ -12,9 +12,12 @@
 //                    digit-reversed positions, output is in natural order so rows leave
 //                    LDS as contiguous float4 stores.
 // Inter-pass twiddles come from two small per-plan tables (float64-computed, read through
-// L1): tw0[(k0-1)*(N/R0) + j] = w_N^(k0*j), tw1[(k1-1)*R2 + n2] = w_N^(R0*k1*n2).
+// L1): tw0[j*R0 + k0] = w_N^(k0*j), tw1[n2*R1 + k1] = w_N^(R0*k1*n2) -- the factors of one
+// butterfly are neighbours in memory (entry 0 of each group is 1 and never read), so a thread
+// fetches them with 16-byte loads at constant offsets from one address.
 #include "sfno_internal.h"
 
+#include <algorithm>
 #include <cmath>
 #include <vector>
 
@@ -177,6 +180,31 @@ __device__ __forceinline__ float4 load4(const void* base, int64_t idx) {
     }
     return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + idx);
 }
+// A tile's input as it sits in registers between its request and its use: four floats, or four bfloat16 in two words.
+template <bool BF16>
+struct Raw4 {
+    using type = float4;
+};
+template <>
+struct Raw4<true> {
+    using type = uint2;
+};
+template <bool BF16>
+__device__ __forceinline__ typename Raw4<BF16>::type load_raw4(const void* base, int64_t idx) {
+    if constexpr (BF16)
+        return *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(base) + idx);
+    else
+        return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + idx);
+}
+__device__ __forceinline__ float4 widen4(float4 v) { return v; }
+__device__ __forceinline__ float4 widen4(uint2 v) {
+    return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+// Marks the point up to which a requested value stays untouched in its registers: without it the compiler moves the
+// register shuffles of the consumer up to the request and waits for the data there, before the work it should overlap.
+__device__ __forceinline__ void use_here(float4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+__device__ __forceinline__ void use_here(uint2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+
 __device__ __forceinline__ unsigned bf16_rne(float f) {
     unsigned u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;      // NaN stays NaN
@@ -204,15 +232,40 @@ __device__ __forceinline__ bool map_block(int nlat, int ngroups, int& lat, int& 
     return lat < nlat;
 }
 
-// ---- forward: decimation in frequency ---------------------------------------------------------------
+// Twiddle look-up of the passes.  TL = false: the per-plan tables in global memory, factors of one butterfly adjacent
+// (tw0[j * R0 + r], tw1[n2 * R1 + r]).  TL = true: copies in LDS, one slab per factor index so that neighbouring lanes
+// read neighbouring words (tw0[(r - 1) * NB + j], tw1[(r - 1) * R2 + n2]); see lds_tables.
+template <bool TL, int R, int NJ>
+__device__ __forceinline__ float2 twiddle(const float2* __restrict__ tw, int j, int r) {
+    return TL ? tw[(r - 1) * NJ + j] : tw[j * R + r];
+}
+
+// Butterfly index of thread `tid` in round `it` of a pass with TOT butterflies.  A last, partial round is not given to the
+// first wavefronts again but to those that idle in the pass with the fewest butterflies (1440 points, four sequences,
+// eight wavefronts: 360 / 576 / 640 butterflies; the 64 + 128 left over go to wavefronts 6 and 7, whose SIMDs have no
+// share in the first pass), which evens out the load of the four SIMDs.
 template <int N, int R0, int R1, int R2, int S, int FT>
+struct PassRounds {
+    static constexpr int RL = (R2 > 1) ? R2 : R1;
+    static constexpr int T0 = S * (N / R0), T1 = (R2 > 1) ? S * (N / R1) : T0, T2 = S * (N / RL);
+    static constexpr int TMIN = T0 < T1 ? (T0 < T2 ? T0 : T2) : (T1 < T2 ? T1 : T2);
+    static constexpr int ROT = TMIN < FT ? (((TMIN + 63) / 64) % (FT / 64)) * 64 : 0;
+    template <int TOT>
+    static __device__ __forceinline__ int index(int tid, int it) {
+        if ((it + 1) * FT > TOT && it > 0 && ROT > 0) return it * FT + ((tid + FT - ROT) & (FT - 1));
+        return it * FT + tid;
+    }
+};
+
+// ---- forward: decimation in frequency ---------------------------------------------------------------
+template <int N, int R0, int R1, int R2, int S, int FT, bool TL = false>
 __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
     using G = Geo<N, R0, R1, R2>;
     {
         constexpr int NB = N / R0, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 float2* base = z + p * G::PITCH + j;
@@ -222,7 +275,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
                 dft<R0, 0>(v);
                 base[0] = v[0];
 #pragma unroll
-                for (int r = 1; r < R0; ++r) base[r * NB] = cmul(v[r], tw0[(r - 1) * NB + j]);
+                for (int r = 1; r < R0; ++r) base[r * NB] = cmul(v[r], twiddle<TL, R0, NB>(tw0, j, r));
             }
         }
     }
@@ -231,7 +284,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
         constexpr int NB = N / R1, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 const int k0 = j / R2, n2 = j - k0 * R2;
@@ -242,7 +295,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
                 dft<R1, 0>(v);
                 base[0] = v[0];
 #pragma unroll
-                for (int r = 1; r < R1; ++r) base[r * R2] = cmul(v[r], tw1[(r - 1) * R2 + n2]);
+                for (int r = 1; r < R1; ++r) base[r * R2] = cmul(v[r], twiddle<TL, R1, R2>(tw1, n2, r));
             }
         }
         __syncthreads();
@@ -252,7 +305,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
         constexpr int NB = N / RL, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 float2* base = z + p * G::PITCH + j * RL;
@@ -269,7 +322,7 @@ __device__ __forceinline__ void passes_dif(float2* z, const float2* __restrict__
 }
 
 // ---- inverse: decimation in time -------------------------------------------------------------------------
-template <int N, int R0, int R1, int R2, int S, int FT>
+template <int N, int R0, int R1, int R2, int S, int FT, bool TL = false>
 __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__ tw0, const float2* __restrict__ tw1, int tid) {
     using G = Geo<N, R0, R1, R2>;
     {
@@ -277,7 +330,7 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
         constexpr int NB = N / RL, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 float2* base = z + p * G::PITCH + j * RL;
@@ -295,7 +348,7 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
         constexpr int NB = N / R1, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 const int k0 = j / R2, n2 = j - k0 * R2;
@@ -303,7 +356,7 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
                 float2 v[R1];
                 v[0] = base[0];
 #pragma unroll
-                for (int r = 1; r < R1; ++r) v[r] = cmul_tw<1>(base[r * R2], tw1[(r - 1) * R2 + n2]);
+                for (int r = 1; r < R1; ++r) v[r] = cmul_tw<1>(base[r * R2], twiddle<TL, R1, R2>(tw1, n2, r));
                 dft<R1, 1>(v);
 #pragma unroll
                 for (int r = 0; r < R1; ++r) base[r * R2] = v[r];
@@ -315,14 +368,14 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
         constexpr int NB = N / R0, TOT = S * NB;
 #pragma unroll
         for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
+            const int e = PassRounds<N, R0, R1, R2, S, FT>::template index<TOT>(tid, it);
             if (e < TOT) {
                 const int p = e / NB, j = e - p * NB;
                 float2* base = z + p * G::PITCH + j;
                 float2 v[R0];
                 v[0] = base[0];
 #pragma unroll
-                for (int r = 1; r < R0; ++r) v[r] = cmul_tw<1>(base[r * NB], tw0[(r - 1) * NB + j]);
+                for (int r = 1; r < R0; ++r) v[r] = cmul_tw<1>(base[r * NB], twiddle<TL, R0, NB>(tw0, j, r));
                 dft<R0, 1>(v);
 #pragma unroll
                 for (int r = 0; r < R0; ++r) base[r * NB] = v[r];
@@ -332,156 +385,353 @@ __device__ __forceinline__ void passes_dit(float2* z, const float2* __restrict__
     __syncthreads();
 }
 
-// grid = 8 * ceil(nlat/8) * ngroups workgroups, ngroups = ceil((ld/4) / S), see map_block
-template <int N, int R0, int R1, int R2, int S, int FT, bool BF16>
-__global__ __launch_bounds__(FT) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const void* __restrict__ x,
-                                                       float* __restrict__ xm, int64_t rows, int nlat, int mmax, int ld, int ngroups, float scale) {
-    using G = Geo<N, R0, R1, R2>;
-    __shared__ __align__(16) float2 z[S * G::PITCH];
-    const int tid = threadIdx.x;
-    int lat, group;
-    if (!map_block(nlat, ngroups, lat, group)) return;
-    const int pair0 = group * S;
-    {
-        // all global loads of the workgroup are issued before the first LDS store
-        constexpr int Q = N / 4, TOT = S * Q, IT = (TOT + FT - 1) / FT;
-        float4 a[IT], b[IT];
-#pragma unroll
-        for (int it = 0; it < IT; ++it) {
-            const int e = tid + it * FT;
-            const int p = e / Q, i4 = e - p * Q;
-            const int64_t r0 = 2 * (int64_t)(pair0 + p);
-            a[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-            b[it] = a[it];
-            if (e < TOT && r0 < rows) a[it] = load4<BF16>(x, (r0 * nlat + lat) * N + 4 * i4);
-            if (e < TOT && r0 + 1 < rows) b[it] = load4<BF16>(x, ((r0 + 1) * nlat + lat) * N + 4 * i4);
-        }
-#pragma unroll
-        for (int it = 0; it < IT; ++it) {
-            const int e = tid + it * FT;
-            if (e < TOT) {
-                const int p = e / Q, i4 = e - p * Q;
-                float4* dst = reinterpret_cast<float4*>(z + p * G::PITCH + 4 * i4);
-                dst[0] = make_float4(a[it].x, b[it].x, a[it].y, b[it].y);
-                dst[1] = make_float4(a[it].z, b[it].z, a[it].w, b[it].w);
-            }
-        }
-    }
-    __syncthreads();
-    passes_dif<N, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
-    const int npairs_ld = ld / 4;
-    const float h = 0.5f * scale;
-    for (int e = tid; e < S * mmax; e += FT) {
-        const int m = e / S, p = e - m * S;
-        if (pair0 + p >= npairs_ld) continue;
-        const float2 zp = z[p * G::PITCH + G::pos(m)];
-        const float2 zq = z[p * G::PITCH + G::pos(m == 0 ? 0 : N - m)];
-        float4 o;
-        o.x = h * (zp.x + zq.x);
-        o.y = h * (zp.y - zq.y);
-        o.z = h * (zp.y + zq.y);
-        o.w = -h * (zp.x - zq.x);
-        *reinterpret_cast<float4*>(xm + ((int64_t)m * nlat + lat) * ld + 4 * (int64_t)(pair0 + p)) = o;
-    }
+// Order handled by thread group u (0 <= u < MP) of a sweep over MP consecutive orders.  With R0 = 16 and four channel
+// pairs per workgroup a wavefront serves 16 orders; bits 3 and 4 of u are swapped so that these are two runs of eight
+// consecutive orders 16 apart: their slots k0 * (N / 16) + k1 * R2 + k2 then fall on all LDS bank pairs evenly
+// (eight consecutive k0 at two consecutive k1), where 16 consecutive orders would share half of them.
+template <int R0, int S, int MP>
+__device__ __forceinline__ int sweep_order(int u) {
+    if constexpr (R0 == 16 && S == 4 && MP >= 32) return (u & ~0x18) | ((u & 8) << 1) | ((u & 16) >> 1);
+    return u;
 }
 
-template <int N, int R0, int R1, int R2, int S, int FT, bool BF16>
-__global__ __launch_bounds__(FT) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const float* __restrict__ xm,
-                                                        void* __restrict__ x, int64_t rows, int nlat, int mmax, int ld, int ngroups,
-                                                        float2* __restrict__ lat_stats) {
+// ---- longitude kernels ---------------------------------------------------------------------------------------
+// Persistent workgroups: the grid holds as many workgroups as the chip keeps resident (two per CU), and each walks the
+// tiles (latitude, group of S channel pairs) of its XCD in steps of the XCD's workgroup count, so that workgroups
+// running at the same time work on neighbouring groups of the same latitudes and the 64-byte pieces they exchange
+// with the order-major buffer meet in that XCD's L2 as whole lines.  The input of the next tile is requested into
+// registers as soon as the current one has been copied to LDS and arrives while the passes run.  Between that request
+// and its use no other value may come from global memory (loads return in order: waiting for a later one waits for
+// the tile as well), so the inter-pass twiddles and the slot table are copied to LDS once per workgroup.
+template <int N, int R0, int R1, int R2>
+struct LdsTables {
+    static constexpr int NB = N / R0;
+    static constexpr int NTW1 = (R2 > 1) ? (R1 - 1) * R2 : 1;
+    float2 tw0[(R0 - 1) * NB];
+    float2 tw1[NTW1];
+    unsigned post[N / 2 + 1];
+};
+
+template <int N, int R0, int R1, int R2, int FT>
+__device__ __forceinline__ void lds_tables(LdsTables<N, R0, R1, R2>& t, const float2* __restrict__ tw0, const float2* __restrict__ tw1,
+                                           const unsigned* __restrict__ post, int tid) {
+    constexpr int NB = N / R0;
+    for (int i = tid; i < (R0 - 1) * NB; i += FT) {
+        const int r = i / NB, j = i - r * NB;
+        t.tw0[i] = tw0[j * R0 + r + 1];
+    }
+    if constexpr (R2 > 1)
+        for (int i = tid; i < (R1 - 1) * R2; i += FT) {
+            const int r = i / R2, n2 = i - r * R2;
+            t.tw1[i] = tw1[n2 * R1 + r + 1];
+        }
+    for (int i = tid; i <= N / 2; i += FT) t.post[i] = post[i];
+}
+
+// tile -> (latitude, first channel pair); tiles of XCD x are the groups of latitudes x, x + 8, ... in that order
+struct TileWalk {
+    int xcd, step, ntiles, ngroups;
+    __device__ __forceinline__ TileWalk(int nlat, int ngroups_) : ngroups(ngroups_) {
+        xcd = blockIdx.x & 7;
+        step = gridDim.x >> 3;
+        ntiles = ((nlat - xcd + 7) >> 3) * ngroups_;
+    }
+    __device__ __forceinline__ int first() const { return blockIdx.x >> 3; }
+    __device__ __forceinline__ void locate(int t, int& lat, int& group) const {
+        const int q = t / ngroups;
+        lat = q * 8 + xcd;
+        group = t - q * ngroups;
+    }
+};
+
+// A tile is one latitude and S * H channel pairs: H = 2 batches of S = 4 pairs for the long rows, one batch of 8 for the
+// shorter ones, so that per order a tile owns one whole 128-byte line of the order-major buffer (8 pairs x 16 bytes).
+// Lines written or read in halves by different workgroups cost a third of the achievable bandwidth here (the two halves
+// reach memory as separate partial-line transactions), so the forward kernel keeps the first batch's results in
+// registers and stores both halves together, and the inverse kernel requests both halves together.
+//
+// grid = 8 * (workgroups per XCD) workgroups, see go_fast
+template <int N, int R0, int R1, int R2, int S, int H, int FT, bool BF16>
+__global__ __launch_bounds__(FT, 4) void rfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const unsigned* __restrict__ post,
+                                                          const void* __restrict__ x, float* __restrict__ xm, int64_t rows, int nlat, int mmax, int ld,
+                                                          int ngroups, float scale) {
     using G = Geo<N, R0, R1, R2>;
-    static_assert(N % 2 == 0, "even length");
-    static_assert(FT % S == 0 && 64 % S == 0, "a thread serves one channel pair");
+    static_assert((S & (S - 1)) == 0 && FT % S == 0 && N % 4 == 0, "a power-of-two number of channel pairs shares the threads evenly");
+    static_assert(H == 1 || H == 2, "one or two batches per tile");
     __shared__ __align__(16) float2 z[S * G::PITCH];
-    __shared__ float4 red[FT / 64][S];
+    __shared__ LdsTables<N, R0, R1, R2> tab;
     const int tid = threadIdx.x;
-    // moments of the output row over longitude, from the coefficients on their way in (lat_stats != null): the mean is
-    // Re X_0, the mean squared deviation from it 2 sum_{0<m<N/2} |X_m|^2 + (Re X_{N/2})^2; (A, B) = the two channels of the pair
-    float mean_a = 0.f, mean_b = 0.f, dev_a = 0.f, dev_b = 0.f;
-    int lat, group;
-    if (!map_block(nlat, ngroups, lat, group)) return;
-    const int pair0 = group * S;
-    const int npairs_ld = ld / 4;
-    constexpr int HALF = N / 2;
-    {
-        // batches of global loads first, then the scatter into digit-reversed LDS slots
-        constexpr int TOT = S * (HALF + 1), IT = (TOT + FT - 1) / FT, BATCH = 6;
+    const TileWalk walk(nlat, ngroups);
+    int t = walk.first();
+    if (t >= walk.ntiles) return;
+    lds_tables<N, R0, R1, R2, FT>(tab, tw0, tw1, post, tid);
+    constexpr int TP = FT / S;                          // threads per channel pair
+    constexpr int Q = N / 4, IT = (Q + TP - 1) / TP;
+    constexpr int NSW = (N / 2 + 1 + TP - 1) / TP;      // sweeps of TP orders that cover every order a plan can keep
+    // TP threads walk the two rows of one channel pair in steps of TP groups of four longitudes: one address per thread and
+    // batch, constant offsets after that.  Requests are unconditional (a load under a branch would be waited for at the end
+    // of its branch): rows that do not exist and the groups of four beyond the row's end read a valid address instead and
+    // are zeroed on their way to LDS.
+    const int pl = tid / TP, q0 = tid - pl * TP;
+    typename Raw4<BF16>::type a[IT], b[IT];
+    bool ha = false, hb = false;
+    auto request = [&](int tile, int half) {
+        int lat, group;
+        walk.locate(tile, lat, group);
+        const int64_t r0 = 2 * (int64_t)((group * H + half) * S + pl);
+        ha = r0 < rows;
+        hb = r0 + 1 < rows;
+        const int64_t ia = ((ha ? r0 : 0) * nlat + lat) * N, ib = ((hb ? r0 + 1 : 0) * nlat + lat) * N;
 #pragma unroll
-        for (int it0 = 0; it0 < IT; it0 += BATCH) {
-            float4 v[BATCH];
+        for (int it = 0; it < IT; ++it) {
+            // (a row can be shorter than one step of the TP threads: the fall-back address is the row's start, not the thread's)
+            const bool in = (it + 1) * TP <= Q || q0 + it * TP < Q;
+            const int off = in ? 4 * (q0 + it * TP) : 0;
+            a[it] = load_raw4<BF16>(x, ia + off);
+            b[it] = load_raw4<BF16>(x, ib + off);
+        }
+    };
+    // the requested batch goes to LDS as complex sequences a + i b
+    auto fill = [&]() {
+        float4* dst = reinterpret_cast<float4*>(z + pl * G::PITCH) + 2 * q0;
 #pragma unroll
-            for (int u = 0; u < BATCH; ++u) {
-                const int e = tid + (it0 + u) * FT;
-                const int m = e / S, p = e - m * S;
-                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (it0 + u < IT && e < TOT && m < mmax && pair0 + p < npairs_ld)
-                    v[u] = *reinterpret_cast<const float4*>(xm + ((int64_t)m * nlat + lat) * ld + 4 * (int64_t)(pair0 + p));
+        for (int it = 0; it < IT; ++it) {
+            use_here(a[it]);
+            use_here(b[it]);
+        }
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            if ((it + 1) * TP <= Q || q0 + it * TP < Q) {
+                float4 fa = widen4(a[it]), fb = widen4(b[it]);
+                if (!ha) fa = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (!hb) fb = make_float4(0.f, 0.f, 0.f, 0.f);
+                dst[2 * it * TP] = make_float4(fa.x, fb.x, fa.y, fb.y);
+                dst[2 * it * TP + 1] = make_float4(fa.z, fb.z, fa.w, fb.w);
             }
+        }
+    };
+    const float h = 0.5f * scale;
+    const int pp_ = tid & (S - 1);
+    const int mfirst = sweep_order<R0, S, TP>(tid / S);
+    const float2* zz = z + pp_ * G::PITCH;
+    // Hermitian split: the two channels of a pair from bins m and N - m
+    auto split = [&](int m) {
+        const unsigned pp = tab.post[m];
+        const float2 zp = zz[pp & 0xffffu], zq = zz[pp >> 16];
+        return make_float4(h * (zp.x + zq.x), h * (zp.y - zq.y), h * (zp.y + zq.y), h * (zq.x - zp.x));
+    };
+    const int64_t mstep = (int64_t)TP * nlat * ld;
+    request(t, 0);
+    for (;;) {
+        int lat, group;
+        walk.locate(t, lat, group);
+        const int tn = t + walk.step;
+        const int tq = tn < walk.ntiles ? tn : t;       // the last tile requests itself again: always a request, never a branch around one
+        const int pair = group * H * S + pp_;
+        float* o = xm + ((int64_t)mfirst * nlat + lat) * ld + 4 * (int64_t)pair;
+        fill();
+        if (H == 2)
+            request(t, 1);
+        else
+            request(tq, 0);
+        __syncthreads();
+        passes_dif<N, R0, R1, R2, S, FT, true>(z, tab.tw0, tab.tw1, tid);
+        if constexpr (H == 1) {
+            if (pair < ld / 4) {
 #pragma unroll
-            for (int u = 0; u < BATCH; ++u) {
-                const int e = tid + (it0 + u) * FT;
-                if (it0 + u < IT && e < TOT) {
-                    const int m = e / S, p = e - m * S;
-                    float4 w = v[u];
-                    if (2 * (int64_t)(pair0 + p) + 1 >= rows) w.z = w.w = 0.f;     // padding slot must not leak into its partner
-                    float2* zz = z + p * G::PITCH;
-                    if (m == 0 || m == HALF) {
-                        zz[G::pos(m)] = make_float2(w.x, w.z);                     // C2R: Im of mean and Nyquist bins dropped
-                        if (m == 0) {
-                            mean_a = w.x;
-                            mean_b = w.z;
-                        } else {
-                            dev_a = fmaf(w.x, w.x, dev_a);
-                            dev_b = fmaf(w.z, w.z, dev_b);
-                        }
-                    } else {
-                        zz[G::pos(m)] = make_float2(w.x - w.w, w.y + w.z);
-                        zz[G::pos(N - m)] = make_float2(w.x + w.w, w.z - w.y);
-                        dev_a += 2.f * fmaf(w.x, w.x, w.y * w.y);
-                        dev_b += 2.f * fmaf(w.z, w.z, w.w * w.w);
-                    }
+                for (int u = 0; u < NSW; ++u)
+                    if (mfirst + u * TP < mmax) *reinterpret_cast<float4*>(o + u * mstep) = split(mfirst + u * TP);
+            }
+        } else {
+            float4 first[NSW];
+#pragma unroll
+            for (int u = 0; u < NSW; ++u)
+                if (mfirst + u * TP < mmax) first[u] = split(mfirst + u * TP);
+            __syncthreads();
+            fill();
+            request(tq, 0);
+            __syncthreads();
+            passes_dif<N, R0, R1, R2, S, FT, true>(z, tab.tw0, tab.tw1, tid);
+            const bool va = pair < ld / 4, vb = pair + S < ld / 4;
+#pragma unroll
+            for (int u = 0; u < NSW; ++u) {
+                if (mfirst + u * TP < mmax) {
+                    const float4 second = split(mfirst + u * TP);
+                    if (va) *reinterpret_cast<float4*>(o + u * mstep) = first[u];
+                    if (vb) *reinterpret_cast<float4*>(o + u * mstep + 4 * S) = second;
                 }
             }
         }
+        if (tn >= walk.ntiles) break;
+        __syncthreads();
+        t = tn;
     }
-    if (lat_stats) {
-        // lanes S apart serve the same pair: fold them, one entry per wavefront and pair
+}
+
+// Inverse.  NSWA = sweeps of TP orders that are read from memory (ceil(mmax / TP), chosen by the launcher among the
+// instantiated values; the orders of the remaining sweeps enter as zeros), LS = the per-latitude moments are written.
+// Every global store that follows a request in program order is unconditional: the wait for a requested value counts the
+// memory operations issued after it, and a store under a branch cannot be counted -- the kernel would wait for its
+// stores to be acknowledged before it touches the next tile's input.  So nothing is skipped, it is aliased instead:
+// a pair slot beyond the last pair of the tensor does the work of the last pair once more (same loads, same sequence,
+// same stores of the same values), the missing second channel of an odd row count is a copy of the first and is stored
+// to the first one's row, and the lanes past the end of a row store its last four values again.
+template <int N, int R0, int R1, int R2, int S, int H, int FT, bool BF16, int NSWA, bool LS>
+__global__ __launch_bounds__(FT, 4) void irfft_fast_kernel(const float2* __restrict__ tw0, const float2* __restrict__ tw1, const unsigned* __restrict__ post,
+                                                           const float* __restrict__ xm, void* __restrict__ x, int64_t rows, int nlat, int mmax, int ld,
+                                                           int ngroups, float2* __restrict__ lat_stats) {
+    using G = Geo<N, R0, R1, R2>;
+    static_assert(N % 4 == 0, "even length");
+    static_assert((S & (S - 1)) == 0 && FT % S == 0 && 64 % S == 0, "a thread serves one channel pair");
+    static_assert(H == 1 || H == 2, "one or two batches per tile");
+    __shared__ __align__(16) float2 z[S * G::PITCH];
+    __shared__ LdsTables<N, R0, R1, R2> tab;
+    __shared__ float4 red[FT / 64][S];
+    const int tid = threadIdx.x;
+    const TileWalk walk(nlat, ngroups);
+    int t = walk.first();
+    if (t >= walk.ntiles) return;
+    lds_tables<N, R0, R1, R2, FT>(tab, tw0, tw1, post, tid);
+    constexpr int HALF = N / 2, TP = FT / S;
+    constexpr int NSW = (HALF + 1 + TP - 1) / TP;        // sweeps over the orders 0..N/2
+    static_assert(NSWA >= 1 && NSWA <= NSW, "sweeps that are read");
+    // With few sweeps the coefficients of both batches of a tile are requested together (the two 64-byte halves of each line
+    // in neighbouring requests: whole-line reads); with many, registers only allow one batch ahead.
+    constexpr bool BOTH = H == 2 && NSWA * H <= 6;
+    constexpr int HV = BOTH ? H : 1;
+    const int pp_ = tid & (S - 1);
+    const int mfirst = sweep_order<R0, S, TP>(tid / S);
+    const int pl = tid / TP, q0 = tid - pl * TP;
+    const int last_pair = (int)((rows + 1) / 2) - 1;
+    float2* zz = z + pp_ * G::PITCH;
+    // A thread keeps its pair and walks the orders in sweeps of TP.  Requests are unconditional, see the forward kernel: an
+    // order the plan does not keep reads order 0 instead and is zeroed when it is used.
+    float4 v[HV][NSWA];
+    auto request = [&](int tile, int half) {
+        int lat, group;
+        walk.locate(tile, lat, group);
+        const float* src = xm + (int64_t)lat * ld;
 #pragma unroll
-        for (int off = S; off < 64; off <<= 1) {
-            mean_a += __shfl_xor(mean_a, off, 64);
-            mean_b += __shfl_xor(mean_b, off, 64);
-            dev_a += __shfl_xor(dev_a, off, 64);
-            dev_b += __shfl_xor(dev_b, off, 64);
-        }
-        if ((tid & 63) < S) red[tid >> 6][tid & 63] = make_float4(mean_a, mean_b, dev_a, dev_b);
-    }
-    __syncthreads();
-    if (lat_stats && tid < S) {
-        float4 t = red[0][tid];
+        for (int u = 0; u < NSWA; ++u) {
+            const int m = mfirst + u * TP;
+            const float* row = src + (int64_t)(m < mmax ? m : 0) * nlat * ld;
 #pragma unroll
-        for (int w = 1; w < FT / 64; ++w) {
-            const float4 u = red[w][tid];
-            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
-        }
-        const int64_t r0 = 2 * (int64_t)(pair0 + tid);
-        if (r0 < rows) lat_stats[r0 * nlat + lat] = make_float2(t.x, t.z);
-        if (r0 + 1 < rows) lat_stats[(r0 + 1) * nlat + lat] = make_float2(t.y, t.w);
-    }
-    passes_dit<N, R0, R1, R2, S, FT>(z, tw0, tw1, tid);
-    {
-        constexpr int Q = N / 4, TOT = S * Q;
-#pragma unroll
-        for (int it = 0; it < (TOT + FT - 1) / FT; ++it) {
-            const int e = tid + it * FT;
-            if (e < TOT) {
-                const int p = e / Q, i4 = e - p * Q;
-                const int64_t r0 = 2 * (int64_t)(pair0 + p);
-                const float4* src = reinterpret_cast<const float4*>(z + p * G::PITCH + 4 * i4);
-                const float4 u0 = src[0], u1 = src[1];
-                if (r0 < rows) store4<BF16>(x, (r0 * nlat + lat) * N + 4 * i4, make_float4(u0.x, u0.z, u1.x, u1.z));
-                if (r0 + 1 < rows) store4<BF16>(x, ((r0 + 1) * nlat + lat) * N + 4 * i4, make_float4(u0.y, u0.w, u1.y, u1.w));
+            for (int hh = 0; hh < HV; ++hh) {
+                const int pair = (group * H + half + hh) * S + pp_;
+                v[hh][u] = *reinterpret_cast<const float4*>(row + 4 * (pair < last_pair ? pair : last_pair));
             }
         }
+    };
+    request(t, 0);
+    __syncthreads();                                      // tables
+    for (;;) {
+        int lat, group;
+        walk.locate(t, lat, group);
+        const int tn = t + walk.step;
+        const int tq = tn < walk.ntiles ? tn : t;         // the last tile requests itself again: always a request, never a branch around one
+#pragma unroll
+        for (int hh = 0; hh < H; ++hh) {
+            const int pair0 = (group * H + hh) * S;
+            // moments of the output row over longitude, from the coefficients on their way in (LS): the mean is
+            // Re X_0, the mean squared deviation from it 2 sum_{0<m<N/2} |X_m|^2 + (Re X_{N/2})^2; (A, B) = the two channels of the pair
+            float mean_a = 0.f, mean_b = 0.f, dev_a = 0.f, dev_b = 0.f;
+            {
+                // Hermitian extension into the slots the decimation-in-time passes expect
+                const int pe = pair0 + pp_ < last_pair ? pair0 + pp_ : last_pair;
+                const bool hb = 2 * (int64_t)pe + 1 < rows;       // odd row count: the second channel of the last pair is a copy of the first
+                float4(&vv)[NSWA] = v[BOTH ? hh : 0];
+#pragma unroll
+                for (int u = 0; u < NSWA; ++u) use_here(vv[u]);
+#pragma unroll
+                for (int u = 0; u < NSW; ++u) {
+                    const int m = mfirst + u * TP;
+                    if (m <= HALF) {
+                        const unsigned pp = tab.post[m];
+                        float4 w = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (u < NSWA) {
+                            w = vv[u < NSWA ? u : 0];
+                            if (m >= mmax) w = make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (!hb) {
+                                w.z = w.x;
+                                w.w = w.y;
+                            }
+                        }
+                        if (m == 0 || m == HALF) {
+                            zz[pp & 0xffffu] = make_float2(w.x, w.z);                  // C2R: Im of mean and Nyquist bins dropped
+                            if (m == 0) {
+                                mean_a = w.x;
+                                mean_b = w.z;
+                            } else {
+                                dev_a = fmaf(w.x, w.x, dev_a);
+                                dev_b = fmaf(w.z, w.z, dev_b);
+                            }
+                        } else {
+                            zz[pp & 0xffffu] = make_float2(w.x - w.w, w.y + w.z);
+                            zz[pp >> 16] = make_float2(w.x + w.w, w.z - w.y);
+                            if (LS && u < NSWA) {
+                                dev_a += 2.f * fmaf(w.x, w.x, w.y * w.y);
+                                dev_b += 2.f * fmaf(w.z, w.z, w.w * w.w);
+                            }
+                        }
+                    }
+                }
+            }
+            if constexpr (LS) {
+                // lanes S apart serve the same pair: fold them, one entry per wavefront and pair
+#pragma unroll
+                for (int off = S; off < 64; off <<= 1) {
+                    mean_a += __shfl_xor(mean_a, off, 64);
+                    mean_b += __shfl_xor(mean_b, off, 64);
+                    dev_a += __shfl_xor(dev_a, off, 64);
+                    dev_b += __shfl_xor(dev_b, off, 64);
+                }
+                if ((tid & 63) < S) red[tid >> 6][tid & 63] = make_float4(mean_a, mean_b, dev_a, dev_b);
+            }
+            __syncthreads();
+            if constexpr (LS) {
+                if (tid < S) {
+                    float4 s4 = red[0][tid];
+#pragma unroll
+                    for (int w = 1; w < FT / 64; ++w) {
+                        const float4 u = red[w][tid];
+                        s4.x += u.x; s4.y += u.y; s4.z += u.z; s4.w += u.w;
+                    }
+                    const int pe = pair0 + tid < last_pair ? pair0 + tid : last_pair;
+                    const int64_t ra = 2 * (int64_t)pe, rb = ra + 1 < rows ? ra + 1 : ra;
+                    lat_stats[ra * nlat + lat] = make_float2(s4.x, s4.z);
+                    lat_stats[rb * nlat + lat] = make_float2(s4.y, s4.w);
+                }
+            }
+            // the next batch's coefficients (after the stores above, so that only unconditional stores follow the request)
+            if constexpr (BOTH) {
+                if (hh == H - 1) request(tq, 0);
+            } else {
+                if (hh < H - 1)
+                    request(t, hh + 1);
+                else
+                    request(tq, 0);
+            }
+            passes_dit<N, R0, R1, R2, S, FT, true>(z, tab.tw0, tab.tw1, tid);
+            {
+                // rows leave LDS in natural order: TP threads walk the two rows of one channel pair, constant offsets from one address
+                constexpr int Q = N / 4, ITS = (Q + TP - 1) / TP;
+                const int pe = pair0 + pl < last_pair ? pair0 + pl : last_pair;
+                const int64_t ra = 2 * (int64_t)pe, rb = ra + 1 < rows ? ra + 1 : ra;
+                const float4* src = reinterpret_cast<const float4*>(z + pl * G::PITCH);
+#pragma unroll
+                for (int it = 0; it < ITS; ++it) {
+                    int i4 = q0 + it * TP;
+                    if ((it + 1) * TP > Q) i4 = i4 < Q ? i4 : Q - 1;
+                    const float4 u0 = src[2 * i4], u1 = src[2 * i4 + 1];
+                    store4<BF16>(x, (ra * nlat + lat) * N + 4 * i4, make_float4(u0.x, u0.z, u1.x, u1.z));
+                    store4<BF16>(x, (rb * nlat + lat) * N + 4 * i4, make_float4(u0.y, u0.w, u1.y, u1.w));
+                }
+            }
+            if (hh < H - 1) __syncthreads();
+        }
+        if (tn >= walk.ntiles) break;
+        __syncthreads();
+        t = tn;
     }
 }
 
@@ -600,19 +850,36 @@ const FastEntry* find_fast(int n) {
 
 template <int N, int R0, int R1, int R2, bool BF16>
 int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t rows, int nlat, int mmax, int ld, float2* lat_stats, hipStream_t s) {
-    constexpr int S = (N >= 1024) ? 4 : 8;
+    constexpr int S = (N >= 1024) ? 4 : 8;              // channel pairs in LDS at a time
+    constexpr int H = 8 / S;                            // batches per tile: a tile owns 8 pairs = one 128-byte line per order
     constexpr int FT = (S * N >= 4096) ? 512 : 256;     // threads per workgroup
-    const int ngroups = (ld / 4 + S - 1) / S;
-    const int64_t nblocks = (int64_t)((nlat + 7) / 8) * ngroups * 8;
-    if (nblocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    dim3 grid((unsigned)nblocks);
+    const int ngroups = (ld / 4 + S * H - 1) / (S * H);
+    // two resident workgroups per CU, the same number on every XCD; fewer when an XCD has fewer tiles than that
+    const int64_t tiles_xcd = (int64_t)((nlat + 7) / 8) * ngroups;
+    const int per_xcd = (int)std::min<int64_t>(tiles_xcd, std::max(1, 2 * p.n_cu / 8));
+    dim3 grid((unsigned)(8 * per_xcd));
     if (!inverse) {
         float scale = (float)(kTwoPi / (double)N);
-        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, in, reinterpret_cast<float*>(out),
-                           rows, nlat, mmax, ld, ngroups, scale);
+        hipLaunchKernelGGL((rfft_fast_kernel<N, R0, R1, R2, S, H, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, p.d_post, in,
+                           reinterpret_cast<float*>(out), rows, nlat, mmax, ld, ngroups, scale);
     } else {
-        hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, FT, BF16>), grid, dim3(FT), 0, s, p.d_tw0, p.d_tw1, reinterpret_cast<const float*>(in), out,
-                           rows, nlat, mmax, ld, ngroups, lat_stats);
+        // sweeps of FT / S orders the kernel reads: all of 0..N/2, or a third of them for truncated plans.  Only the truncated
+        // plans afford the registers to request both batches of a tile at once (whole-line reads); the others walk tiles of one
+        // batch, whose finer grain also leaves a shorter tail when the tiles do not divide evenly among the workgroups.
+        constexpr int TP = FT / S, NSW = (N / 2 + 1 + TP - 1) / TP, NSMALL = (NSW + 2) / 3;
+        const float* xm = reinterpret_cast<const float*>(in);
+        const bool small = mmax <= NSMALL * TP;
+        const int ng = small ? ngroups : (ld / 4 + S - 1) / S;
+        const int per = (int)std::min<int64_t>((int64_t)((nlat + 7) / 8) * ng, std::max(1, 2 * p.n_cu / 8));
+#define IRFFT_GO(H_, NSWA_, LS_)                                                                                                            \
+    hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, H_, FT, BF16, NSWA_, LS_>), dim3((unsigned)(8 * per)), dim3(FT), 0, s, p.d_tw0, \
+                       p.d_tw1, p.d_post, xm, out, rows, nlat, mmax, ld, ng, lat_stats)
+        if (lat_stats) {
+            if (small) IRFFT_GO(H, NSMALL, true); else IRFFT_GO(1, NSW, true);
+        } else {
+            if (small) IRFFT_GO(H, NSMALL, false); else IRFFT_GO(1, NSW, false);
+        }
+#undef IRFFT_GO
     }
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
@@ -651,18 +918,26 @@ int go_chirp(bool inverse, const FftPlan& p, const float* in, float* out, int mm
 // inter-pass twiddles of the specialised passes of length f.n
 int upload_pass_twiddles(const FastEntry& f, FftPlan& p) {
     const int N = f.n, nb = N / f.r0;
-    std::vector<float2> tw0((size_t)(f.r0 - 1) * nb), tw1((size_t)std::max(1, (f.r1 - 1) * f.r2));
+    std::vector<float2> tw0((size_t)f.r0 * nb, make_float2(1.f, 0.f)), tw1((size_t)std::max(1, f.r1 * f.r2), make_float2(1.f, 0.f));
     for (int k0 = 1; k0 < f.r0; ++k0)
         for (int j = 0; j < nb; ++j) {
             double a = -kTwoPi * (double)(((int64_t)k0 * j) % N) / (double)N;
-            tw0[(size_t)(k0 - 1) * nb + j] = make_float2((float)std::cos(a), (float)std::sin(a));
+            tw0[(size_t)j * f.r0 + k0] = make_float2((float)std::cos(a), (float)std::sin(a));
         }
-    tw1[0] = make_float2(1.f, 0.f);
     for (int k1 = 1; k1 < f.r1; ++k1)
         for (int n2 = 0; n2 < f.r2; ++n2) {
             double a = -kTwoPi * (double)(((int64_t)f.r0 * k1 * n2) % N) / (double)N;
-            tw1[(size_t)(k1 - 1) * f.r2 + n2] = make_float2((float)std::cos(a), (float)std::sin(a));
+            tw1[(size_t)n2 * f.r1 + k1] = make_float2((float)std::cos(a), (float)std::sin(a));
         }
+    // slots of bin m and of bin N - m after the decimation-in-frequency passes (= before the decimation-in-time passes)
+    std::vector<unsigned> post((size_t)N / 2 + 1);
+    auto slot = [&](int m) {
+        const int k0 = m % f.r0, t = m / f.r0, k1 = t % f.r1, k2 = t / f.r1;
+        return (unsigned)(k0 * (f.r1 * f.r2) + k1 * f.r2 + k2);
+    };
+    for (int m = 0; m <= N / 2; ++m) post[m] = slot(m) | (slot((N - m) % N) << 16);
+    if (hipMalloc(&p.d_post, sizeof(unsigned) * post.size()) != hipSuccess) return SFNO_ENOMEM;
+    if (hipMemcpy(p.d_post, post.data(), sizeof(unsigned) * post.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;
     if (hipMalloc(&p.d_tw0, sizeof(float2) * tw0.size()) != hipSuccess) return SFNO_ENOMEM;
     if (hipMalloc(&p.d_tw1, sizeof(float2) * tw1.size()) != hipSuccess) return SFNO_ENOMEM;
     if (hipMemcpy(p.d_tw0, tw0.data(), sizeof(float2) * tw0.size(), hipMemcpyHostToDevice) != hipSuccess) return SFNO_EHIP;

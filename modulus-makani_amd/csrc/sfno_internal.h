@@ -125,11 +125,13 @@ int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_wo
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
 struct FftPlan {
     int n = 0;                     // transform length (nlon)
+    int n_cu = 256;                // compute units of the plan's device (sizes the persistent grids of fft_fast.hip)
     int npass = 0;
     int radix[24];
     float2* d_tw = nullptr;        // [n] exp(-2 pi i j / n)
     float2* d_tw0 = nullptr;       // inter-pass twiddles of the specialised kernels (fft_fast.hip)
     float2* d_tw1 = nullptr;
+    unsigned* d_post = nullptr;    // [n/2+1] LDS slot of bin m (low half) and of bin n - m (high half) around the specialised passes
     // latitude plans of lengths with a large prime factor (fft_chirp_plan_init): the DFT as a circular convolution of
     // length chirp_m with a chirp; d_tw0 / d_tw1 then belong to the specialised passes of length chirp_m
     int chirp_m = 0;

@@ -74,6 +74,19 @@ def packed_for(weight, compute="fp32", adjoint=False):
     return p.refresh(weight, adjoint)
 
 
+def clear_cache(weight=None):
+    """Forgets the packed copies of `weight` (of every weight if None), so that the next call packs the parameter again.
+
+    The cache notices in-place updates through the tensor's version counter (optimizer steps, ``copy_`` under
+    ``no_grad``).  Writes through ``param.data`` (``p.data.add_()``, EMA swaps, some fused optimizers) do not move that
+    counter: call this, or ``SpectralConv.invalidate_packed()``, after such a write."""
+    if weight is None:
+        _cache.clear()
+        return
+    for key in [k for k in _cache if k[0] == id(weight)]:
+        _cache.pop(key, None)
+
+
 def _stream(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
@@ -81,6 +94,8 @@ def _stream(device):
 def _weight_grad(spec_in, gspec_out, shape, batch, mmax, triangular):
     """gw[i,o,l] = sum_{b,m} conj(x[b,i,l,m]) g[b,o,l,m] from spectral-layout buffers."""
     I, O, L = shape
+    if batch == 0:
+        return torch.zeros((I, O, L), dtype=torch.complex64, device=spec_in.device)
     gw = torch.empty((I, O, L), dtype=torch.complex64, device=spec_in.device)
     check(
         lib.sfno_dhconv_weight_grad(I, O, L, ctypes.c_void_p(spec_in.data_ptr()), ctypes.c_void_p(gspec_out.data_ptr()),
@@ -123,6 +138,8 @@ def _dhconv_spectral(spec_in, weight, batch, mmax, triangular, compute, adjoint)
     out = torch.empty((mmax, L, ld_out), dtype=torch.float32, device=spec_in.device)
     if ld_out != 2 * batch * O:
         out.zero_()
+    if batch == 0:
+        return out
     s = ctypes.c_void_p(torch.cuda.current_stream(spec_in.device).cuda_stream)
     check(
         lib.sfno_dhconv_spectral(pw.handle, ctypes.c_void_p(spec_in.data_ptr()), ctypes.c_void_p(out.data_ptr()), batch, mmax, int(triangular), s),

@@ -44,6 +44,15 @@ def packed_weight(weight):
     return p
 
 
+def clear_cache(weight=None):
+    """Forgets the packed copy of `weight` (of every weight if None); needed only after writes through ``param.data``, which
+    the version stamp of the cache does not see."""
+    if weight is None:
+        _wcache.clear()
+    else:
+        _wcache.pop(id(weight), None)
+
+
 def supported(x):
     """Whether the fused kernels take this activation tensor."""
     return x.is_cuda and x.dim() == 4 and x.dtype == torch.bfloat16 and (x.shape[2] * x.shape[3]) % 8 == 0 and x.shape[2] * x.shape[3] >= 8

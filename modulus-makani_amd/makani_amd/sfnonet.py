@@ -139,8 +139,11 @@ class FourierNeuralOperatorBlock(nn.Module):
     def __init__(self, forward_transform, inverse_transform, embed_dim, filter_type="linear", operator_type="diagonal", mlp_ratio=2.0,
                  mlp_drop_rate=0.0, path_drop_rate=0.0, act_layer=nn.GELU, norm_layer=(nn.Identity, nn.Identity), rank=1.0, factorization=None,
                  separable=False, inner_skip="linear", outer_skip=None, use_mlp=False, complex_activation="real", spectral_layers=1, bias=False,
-                 final_activation=False, **kwargs):
+                 final_activation=False, fused_pointwise=True, **kwargs):
         super().__init__()
+        # fused_pointwise (not a Makani option): evaluate the tail of the block with the fused HIP kernels when no gradient
+        # is recorded and the activations are bfloat16; False keeps the PyTorch modules in every situation
+        self.fused_pointwise = fused_pointwise
         if path_drop_rate > 0.0:
             raise NotImplementedError("stochastic depth is a training feature outside this path")
         self.input_shape_loc = (forward_transform.nlat, forward_transform.nlon)
@@ -236,8 +239,14 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                  encoder_layers=1, pos_embed="none", pos_drop_rate=0.0, path_drop_rate=0.0, mlp_drop_rate=0.0,
                  normalization_layer="instance_norm", max_modes=None, hard_thresholding_fraction=1.0, big_skip=True, rank=1.0,
                  factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0,
-                 spectral_compute="fp32", **kwargs):
+                 spectral_compute="fp32", fused_pointwise=True, **kwargs):
         super().__init__()
+        # fused_pointwise (not a Makani option): under torch.no_grad() / inference_mode() with bf16 autocast the 1x1 convolutions,
+        # instance norms and GELUs run on the fused HIP kernels (weights rounded to bf16 once, fp32 accumulation, one rounding per
+        # layer, norm0 statistics from the unrounded field).  A forward that records gradients always runs the PyTorch modules, so
+        # a validation pass under no_grad does not follow the training forward's arithmetic to the bit: pass False (or set the
+        # attribute on the network and on every block) where train and validation numbers must come from the same path.
+        self.fused_pointwise = fused_pointwise
         # spectral_compute = "bf16" (not a Makani option) runs the Legendre and dhconv contractions on bf16 MFMA
         self.spectral_compute = spectral_compute
         if spectral_transform not in ("sht", "fft"):
@@ -275,7 +284,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                                            mlp_drop_rate=mlp_drop_rate, path_drop_rate=0.0 if path_drop_rate == 0.0 else path_drop_rate * i / max(num_layers - 1, 1),
                                            act_layer=act, norm_layer=(norm, norm), inner_skip="none", outer_skip="linear", use_mlp=use_mlp, rank=rank,
                                            factorization=factorization, separable=separable, complex_activation=complex_activation,
-                                           spectral_layers=spectral_layers, bias=bias))
+                                           spectral_layers=spectral_layers, bias=bias, fused_pointwise=fused_pointwise))
             self.blocks[-1].filter.filter.compute = spectral_compute
 
         self.decoder = EncoderDecoder(encoder_layers, embed_dim, out_chans, int(decoder_ratio * embed_dim), act, gain=0.5 if big_skip else 1.0)

@@ -139,6 +139,18 @@ class _SHTBase(nn.Module):
             self._plans[key] = p
         return p
 
+    def _adjoint_module(self):
+        """The module whose adjoint plan serves this module's backward pass: the module itself, except for an inverse
+        transform that keeps more orders than the longitude grid resolves (mmax > nlon // 2 + 1).  Such an inverse drops
+        the surplus orders like a complex-to-real FFT does, so their cotangents are exactly zero and the adjoint is that of
+        the same transform truncated to nlon // 2 + 1 orders."""
+        if self.mmax <= self.nlon // 2 + 1 or self._directions != _lib.DIR_INVERSE:
+            return self
+        if getattr(self, "_truncated", None) is None:
+            object.__setattr__(self, "_truncated", type(self)(self.nlat, self.nlon, self.lmax, self.nlon // 2 + 1, self.grid, self.norm, self.csphase,
+                                                              self.compute))
+        return self._truncated
+
     def workspace(self, plan, rows, device):
         nbytes = lib.sfno_sht_workspace_bytes(plan.handle, rows)
         return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
@@ -149,6 +161,7 @@ class _SHTBase(nn.Module):
     def __getstate__(self):
         state = dict(self.__dict__)
         state["_plans"] = {}
+        state.pop("_truncated", None)
         return state
 
     def __deepcopy__(self, memo):
@@ -211,6 +224,8 @@ class _AnalysisFn(torch.autograd.Function):
         g = g.contiguous()
         rows = _rows(ctx.shape[:-2])
         gx = torch.empty(ctx.shape, dtype=torch.bfloat16 if ctx.dt == _lib.DTYPE_BF16 else torch.float32, device=g.device)
+        if rows == 0:
+            return gx, None, None
         plan = mod.plan(g.device, adjoint=True)
         ws, nbytes = mod.workspace(plan, rows, g.device)
         check(lib.sfno_sht_analysis_adjoint(plan.handle, _ptr(g), _ptr(gx), ctx.dt, rows, _ptr(ws), nbytes, _stream_ptr(g.device)),
@@ -229,7 +244,7 @@ class _InverseFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, g):
-        mod = ctx.mod
+        full, mod = ctx.mod, ctx.mod._adjoint_module()
         g = g.float().contiguous()
         lead = g.shape[:-2]
         gc = torch.empty((*lead, mod.lmax, mod.mmax), dtype=torch.complex64, device=g.device)
@@ -238,6 +253,8 @@ class _InverseFn(torch.autograd.Function):
             ws, nbytes = mod.workspace(plan, _rows(lead), g.device)
             check(lib.sfno_sht_inverse_adjoint(plan.handle, _ptr(g), _ptr(gc), _rows(lead), _ptr(ws), nbytes, _stream_ptr(g.device)),
                   "sfno_sht_inverse_adjoint")
+        if mod is not full:      # orders the longitude grid does not resolve receive no gradient
+            gc = torch.nn.functional.pad(gc, (0, full.mmax - mod.mmax))
         return gc, None
 
 
@@ -252,8 +269,10 @@ class _SynthesisFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, g):
-        mod = ctx.mod
+        full, mod = ctx.mod, ctx.mod._adjoint_module()
         rows = _rows(ctx.lead)
+        if rows == 0:
+            return torch.zeros(full.spectral_shape(0), dtype=torch.float32, device=g.device), None, None, None
         plan = mod.plan(g.device, adjoint=True)
         if g.dtype == torch.bfloat16 and lib.sfno_sht_io_dtype_supported(plan.handle, _lib.DTYPE_BF16):
             g, dt = g.contiguous(), _lib.DTYPE_BF16
@@ -263,6 +282,8 @@ class _SynthesisFn(torch.autograd.Function):
         ws, nbytes = mod.workspace(plan, rows, g.device)
         check(lib.sfno_sht_synthesis_adjoint(plan.handle, _ptr(g), dt, _ptr(gspec), rows, _ptr(ws), nbytes, _stream_ptr(g.device)),
               "sfno_sht_synthesis_adjoint")
+        if mod is not full:      # orders the longitude grid does not resolve receive no gradient (the order axis comes first)
+            gspec = torch.cat((gspec, gspec.new_zeros((full.mmax - mod.mmax,) + tuple(gspec.shape[1:]))), dim=0)
         return gspec, None, None, None
 
 
@@ -307,6 +328,8 @@ class RealSHT(_SHTBase):
         plan = self.plan(x.device)
         rows = _rows(x.shape[:-2])
         spec = torch.empty(self.spectral_shape(rows), dtype=torch.float32, device=x.device)
+        if rows == 0:
+            return spec
         ws, nbytes = self.workspace(plan, rows, x.device)
         check(lib.sfno_sht_analysis(plan.handle, _ptr(x), dt, _ptr(spec), rows, _ptr(ws), nbytes, _stream_ptr(x.device)), "sfno_sht_analysis")
         return spec
@@ -361,6 +384,8 @@ class InverseRealSHT(_SHTBase):
         fused = dtype == torch.bfloat16
         out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.bfloat16 if fused else torch.float32, device=spec.device)
         stats = torch.empty((rows, self.nlat, 2), dtype=torch.float32, device=spec.device)
+        if rows == 0:
+            return (out if out.dtype == dtype else out.to(dtype)), stats
         ws, nbytes = self.workspace(plan, rows, spec.device)
         check(lib.sfno_sht_synthesis_lat_stats(plan.handle, _ptr(spec.contiguous()), _ptr(out), _lib.DTYPE_BF16 if fused else _lib.DTYPE_F32, rows,
                                                _ptr(ws), nbytes, _ptr(stats), _stream_ptr(spec.device)), "sfno_sht_synthesis_lat_stats")
@@ -370,6 +395,8 @@ class InverseRealSHT(_SHTBase):
         rows = _rows(lead)
         plan = self.plan(spec.device)
         out = torch.empty((*lead, self.nlat, self.nlon), dtype=torch.bfloat16 if fused else torch.float32, device=spec.device)
+        if rows == 0:
+            return out
         ws, nbytes = self.workspace(plan, rows, spec.device)
         check(lib.sfno_sht_synthesis(plan.handle, _ptr(spec), _ptr(out), _lib.DTYPE_BF16 if fused else _lib.DTYPE_F32, rows, _ptr(ws), nbytes,
                                      _stream_ptr(spec.device)), "sfno_sht_synthesis")

@@ -7,7 +7,7 @@ import math
 import torch
 import torch.nn as nn
 
-from .contractions import get_contract_fun, dhconv_spectral
+from .contractions import get_contract_fun, dhconv_spectral, clear_cache
 from .sht import RealSHT, InverseRealSHT
 
 
@@ -72,6 +72,10 @@ class SpectralConv(nn.Module):
         )
         # coefficients of a spherical transform vanish for l < m; the planar pair fills the whole rectangle
         self._triangular = not getattr(forward_transform, "_planar", False)
+
+    def invalidate_packed(self):
+        """Drops the packed MFMA operand copies of ``weight``; call after writing the parameter through ``.data``."""
+        clear_cache(self.weight)
 
     def forward(self, x, lat_stats=False):
         """Returns (x, residual) as the reference does.  With lat_stats=True (inference on the fused path only) a third value

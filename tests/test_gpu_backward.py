@@ -254,3 +254,42 @@ def test_sfno_training_step_gradients(lib_built):
     assert gmax > 0
     for n in got:
         assert norm(got[n] - want[n]) < 1e-4 * max(norm(want[n]), 1e-2 * gmax), n
+
+
+@pytest.mark.parametrize("spectral", [False, True])
+def test_inverse_with_surplus_orders_backward(lib_built, spectral):
+    """An inverse transform may keep more orders than its longitude grid resolves (mmax > nlon // 2 + 1): the surplus is
+    dropped like a complex-to-real FFT drops it, so its gradient is exactly zero and the rest equals the gradient of the
+    reference op sequence (float64 autograd through the einsum + irfft, which crops the same way)."""
+    import makani_amd as ma
+
+    nlat, nlon, lmax, mmax = 12, 16, 12, 12
+    print(f"case sht-inv-bwd surplus orders {nlat}x{nlon} l{lmax} m{mmax} spectral={spectral}", flush=True)
+    torch.manual_seed(16)
+    mod = ma.InverseRealSHT(nlat, nlon, lmax, mmax, grid="legendre-gauss")
+    ref = TorchRefSHT(nlat, nlon, lmax, mmax, "legendre-gauss", "ortho", directions=("inv",), dtype=torch.float64)
+    c = torch.randn(2, 3, lmax, mmax, dtype=torch.complex64)
+    g = torch.randn(2, 3, nlat, nlon)
+    cr = c.to(torch.complex128).requires_grad_(True)
+    ref.inverse(cr).backward(g.double())
+    cg = c.cuda().requires_grad_(True)
+    if spectral:
+        # the same transform on the order-major layout, as SpectralConv chains it
+        from makani_amd.contractions import _to_spectral
+        from makani_amd._lib import lib, check
+        import ctypes
+
+        spec = _to_spectral(c.cuda().contiguous(), 6, lmax, mmax, True).requires_grad_(True)
+        mod.synthesis(spec, (2, 3)).backward(g.cuda())
+        gs = spec.grad
+        assert tuple(gs.shape) == mod.spectral_shape(6) and float(gs[nlon // 2 + 1:].abs().max()) == 0.0
+        grad = torch.empty(2, 3, lmax, mmax, dtype=torch.complex64, device="cuda")
+        check(lib.sfno_spectral_to_coeffs(ctypes.c_void_p(gs.contiguous().data_ptr()), ctypes.c_void_p(grad.data_ptr()), 6, lmax, mmax, 1,
+                                          ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "to_coeffs")
+    else:
+        mod(cg).backward(g.cuda())
+        grad = cg.grad
+    torch.cuda.synchronize()
+    assert grad.shape == c.shape
+    assert float(grad[..., nlon // 2 + 1:].abs().max()) == 0.0 and float(cr.grad[..., nlon // 2 + 1:].abs().max()) == 0.0
+    assert rel_l2(grad, cr.grad) < TOL

@@ -156,3 +156,49 @@ def test_spectral_conv_diagonal(lib_built):
     ref, _ = spectral_conv(x.double().numpy(), conv.weight.detach().cpu().numpy().astype(np.complex128), t, t)
     assert rel_l2(y.detach().cpu().numpy(), ref) < TOL
     assert torch.equal(res, x.cuda())
+
+
+def test_packed_weight_cache_and_data_writes(lib_built):
+    """The packed operand copy follows in-place updates through the parameter's version counter; a write through ``.data``
+    leaves that counter alone and needs the explicit invalidation hook."""
+    import makani_amd as ma
+    from makani_amd import contractions
+
+    torch.manual_seed(8)
+    ft = ma.RealSHT(16, 32, lmax=16, mmax=17, grid="legendre-gauss")
+    it = ma.InverseRealSHT(16, 32, lmax=16, mmax=17, grid="legendre-gauss")
+    conv = ma.SpectralConv(ft, it, 4, 4, operator_type="dhconv").cuda()
+    x = torch.randn(1, 4, 16, 32).cuda()
+    with torch.no_grad():
+        y0, _ = conv(x)
+        conv.weight.data.mul_(3.0)             # invisible to the cache
+        y_stale, _ = conv(x)
+        conv.invalidate_packed()
+        y1, _ = conv(x)
+        conv.weight.data.mul_(2.0)
+        contractions.clear_cache()             # the module-wide form
+        y2, _ = conv(x)
+    torch.cuda.synchronize()
+    assert torch.equal(y_stale, y0)
+    assert rel_l2(y1.cpu().numpy(), 3 * y0.cpu().numpy()) < 1e-6
+    assert rel_l2(y2.cpu().numpy(), 6 * y0.cpu().numpy()) < 1e-6
+
+
+@pytest.mark.parametrize("updown", [False, True])
+def test_spectral_conv_empty_batch(lib_built, updown):
+    """Batch size 0 returns empty tensors of the right shape, as the reference's einsum path does."""
+    import makani_amd as ma
+
+    ft = ma.RealSHT(33, 64, lmax=16, mmax=17, grid="equiangular") if updown else ma.RealSHT(16, 32, lmax=16, mmax=17, grid="legendre-gauss")
+    it = ma.InverseRealSHT(16, 32, lmax=16, mmax=17, grid="legendre-gauss")
+    conv = ma.SpectralConv(ft, it, 6, 4, operator_type="dhconv").cuda()
+    x = torch.empty(0, 6, ft.nlat, ft.nlon, device="cuda")
+    with torch.no_grad():
+        y, res = conv(x)
+    assert tuple(y.shape) == (0, 4, 16, 32)
+    assert tuple(res.shape) == ((0, 6, 16, 32) if updown else (0, 6, 16, 32))
+    xg = torch.empty(0, 6, ft.nlat, ft.nlon, device="cuda", requires_grad=True)
+    y, _ = conv(xg)
+    y.sum().backward()
+    assert tuple(xg.grad.shape) == tuple(xg.shape) and tuple(conv.weight.grad.shape) == tuple(conv.weight.shape)
+    assert float(conv.weight.grad.abs().max()) == 0.0

@@ -182,3 +182,36 @@ def test_latitude_moments_absent_without_specialised_longitude_kernel(lib_built)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     rc = lib.sfno_sht_synthesis_lat_stats(plan.handle, P(spec), P(out), 0, 4, P(ws), nbytes, P(st), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc == -5
+
+
+@pytest.mark.parametrize("nlat,nlon,lmax,mmax,C", [(721, 1440, 240, 241, 24), (64, 128, 40, 41, 10)])
+def test_latitude_moments_against_statistics_of_the_rounded_field(lib_built, nlat, nlon, lmax, mmax, C):
+    """norm0 on the fused path takes its statistics from the field before it is rounded to bfloat16 (the inverse transform's
+    by-product), the reference's InstanceNorm2d from the rounded tensor it is given.  The means agree (rounding to nearest
+    averages out); the variance of the rounded tensor is larger by the variance of the rounding error, ulp^2 / 12, which is
+    1e-3 of the field's variance for a channel whose mean is ten standard deviations from zero, as in this test.  The
+    normalised outputs of the two conventions therefore differ by a factor 1 +- 6e-4 around the mean: bounded here at 2e-3
+    relative L2 and at 8e-3 (one bfloat16 ulp at one; measured 3.5e-3) in the largest element, in units of the normalised field."""
+    import makani_amd as ma
+    from makani_amd import pointwise as pw
+
+    print(f"case lat-moments vs rounded statistics {nlat}x{nlon} C={C}", flush=True)
+    torch.manual_seed(33)
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid="equiangular")
+    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid="equiangular")
+    field = torch.randn(1, C, nlat, nlon).cuda() + 2.0 * torch.randn(1, C, 1, 1).cuda()
+    with torch.no_grad():
+        spec = sht.analysis(field)
+        x, stats = isht.synthesis_with_lat_stats(spec, (1, C), dtype=torch.bfloat16)
+    gamma, beta = (1.0 + 0.2 * torch.randn(C)).cuda(), torch.randn(C).cuda()
+    sc_l, sh_l = pw.instance_norm_coeffs_lat(stats, 1, gamma, beta, 1e-6)
+    sc_r, sh_r = pw.instance_norm_coeffs(x, gamma, beta, 1e-6)
+    torch.cuda.synchronize()
+    xf = x.float()
+    y_l = (sc_l[:, :, None, None] * xf + sh_l[:, :, None, None] - beta[None, :, None, None]) / gamma[None, :, None, None]
+    y_r = (sc_r[:, :, None, None] * xf + sh_r[:, :, None, None] - beta[None, :, None, None]) / gamma[None, :, None, None]
+    e2 = ((y_l - y_r).norm() / y_r.norm()).item()
+    emax = (y_l - y_r).abs().max().item()
+    mean_gap = ((sh_l - beta) / sc_l - (sh_r - beta) / sc_r).abs().div(xf.std(dim=(2, 3))).max().item()     # difference of the means, in standard deviations
+    print(f"  normalised fields differ by {e2:.2e} (relative L2), {emax:.2e} at most; means by {mean_gap:.2e} standard deviations", flush=True)
+    assert e2 < 2e-3 and emax < 8e-3 and mean_gap < 1e-3

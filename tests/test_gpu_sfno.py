@@ -176,3 +176,27 @@ def test_fused_pointwise_tail_matches_module_path(lib_built):
     with torch.autocast("cuda", dtype=torch.bfloat16):
         y_grad = net(x.cuda().requires_grad_(True))
     assert y_grad.requires_grad
+
+
+def test_fused_pointwise_switch(lib_built):
+    """fused_pointwise=False at construction keeps the PyTorch modules under no_grad + bf16 autocast too: the result equals
+    the one of a network built with the default and switched off attribute by attribute, and differs from the fused one."""
+    case = dict(inp_shape=(33, 64), out_shape=(33, 64), inp_chans=3, out_chans=3, scale_factor=2, embed_dim=16, num_layers=2)
+    torch.manual_seed(4)
+    from makani_amd.sfnonet import SphericalFourierNeuralOperatorNet
+
+    net_off = SphericalFourierNeuralOperatorNet(**case, fused_pointwise=False).cuda().eval()
+    net_on = SphericalFourierNeuralOperatorNet(**case).cuda().eval()
+    net_on.load_state_dict(net_off.state_dict())
+    assert not net_off.fused_pointwise and all(not b.fused_pointwise for b in net_off.blocks)
+    x = torch.randn(2, 3, 33, 64, generator=torch.Generator().manual_seed(5)).cuda()
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y_off, y_on = net_off(x), net_on(x)
+        net_on.fused_pointwise = False
+        for b in net_on.blocks:
+            b.fused_pointwise = False
+        y_on_off = net_on(x)
+    torch.cuda.synchronize()
+    assert torch.equal(y_off, y_on_off)
+    assert not torch.equal(y_off, y_on)
+    assert rel_l2(y_on.float().cpu().numpy(), y_off.float().cpu().numpy()) < 3e-2

@@ -25,7 +25,9 @@ Pinning status (what each function is checked against, see tests/test_oracle_*.p
                             discrete orthonormality, equatorial symmetry.
   sht.sht_forward/inverse : constant field, one-hot Y_l^m samples, band-limited
                             round trip, Parseval, brute-force O(N^2) DFT.
-  dhconv.dhconv           : brute-force loops, identity weights, L=1 matmul.
+  dhconv.dhconv           : brute-force loops (both the einsum and the matrix-product branch), identity weights, L=1 matmul.
+  sfno.SfnoOracle         : an independent evaluation from scipy's harmonics and explicit formulas (tests/test_oracle_sfno_pin.py).
+  stepper.*               : hand-computed statistics and residual rule (tests/test_stepper.py).
   The reference holds no golden vectors for transform values (its tests check shapes
   only), so raw-coefficient sign/ordering conventions of torch-harmonics (latitude
   north->south, Condon-Shortley phase) are "parity unpinned" by reference fixtures;

@@ -24,6 +24,7 @@ for p in (ROOT, os.path.join(ROOT, "modulus-makani_amd")):
         sys.path.insert(0, p)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 
@@ -89,14 +90,38 @@ def make_fields(isht, channels, device):
     return x.contiguous()
 
 
-def read_traffic(key):
-    """HBM bytes per launch from the committed rocprofv3 counter summary, if one exists."""
+def csrc_hash():
+    """sha256 over the kernel and host sources the library is built from (file names and contents, sorted)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "modulus-makani_amd", "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc)) + [os.path.join(ROOT, "include", "sfno_spectral.h")]
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def read_traffic(key, note=None):
+    """HBM bytes per launch from the committed rocprofv3 counter summary -- only if that summary was taken on the kernel
+    sources this run was built from (profiles/traffic.json records their hash); otherwise None, with the reason in `note`."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(key)
+            t = json.load(f)
     except (OSError, ValueError):
         return None
+    entry = t.get(key)
+    if entry is None:
+        return None
+    if not isinstance(entry, dict) or entry.get("csrc_sha") != csrc_hash():
+        if note is not None:
+            note.append(f"profiles/traffic.json[{key}] was measured on other kernel sources "
+                        f"({entry.get('csrc_sha') if isinstance(entry, dict) else 'no hash recorded'} != {csrc_hash()}): not reported")
+        return None
+    return entry.get("bytes")
 
 
 def cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, channels, sample):
@@ -199,9 +224,15 @@ def bench_sht_pair(args):
     else:
         # contraction on the bf16 matrix pipe (fp32 operands cut into three bf16 planes, or bf16 operands): 45 flop per byte is
         # far below that pipe's ridge (312), so HBM is the roofline that bounds the kernel
+        tnote = []
+        # what the matrix pipe executes: half the algorithmic MACs (equator fold), each as six bf16 products (one in bf16 mode)
+        executed = leg_flops / 2 * (6 if args.compute == "fp32" else 1)
         roofline = {"kernel": f"legendre_fold_kernel ({dom})", "bound": "hbm", "achieved": hbm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": hbm_gbs / PEAK_HBM_GBS, "traffic": read_traffic(dom), "algorithmic_bytes_per_launch": leg_bytes,
+                    "frac": hbm_gbs / PEAK_HBM_GBS, "traffic": read_traffic(dom, tnote), "algorithmic_bytes_per_launch": leg_bytes,
                     "avg_launch_ms": stage_ms[dom], "against_fp32_mfma_peak": mfma_view,
+                    "executed_on_bf16_pipe": {"flops_per_launch": executed, "achieved_TFLOPs": executed / (stage_ms[dom] * 1e-3) / 1e12,
+                                              "peak_TFLOPs": PEAK_BF16_MFMA_TFLOPS, "frac": executed / (stage_ms[dom] * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS},
+                    "traffic_note": tnote[0] if tnote else None,
                     "note": ("algorithmic bytes = Fourier panel + triangular table at the reference's element size + triangular coefficients, "
                              "each moved once; the kernel folds the equator (half the MACs and table entries)"
                              + (" and forms every fp32 product from six bf16 MFMA partial products of exactly split operands (6-byte table "
@@ -231,6 +262,8 @@ def bench_sht_pair(args):
         "fft_hbm": {
             "rfft_GBps": fft_bytes / (stage_ms["rfft"] * 1e-3) / 1e9,
             "irfft_GBps": fft_bytes / (stage_ms["irfft"] * 1e-3) / 1e9,
+            "rfft_frac": fft_bytes / (stage_ms["rfft"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+            "irfft_frac": fft_bytes / (stage_ms["irfft"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
             "peak_GBps": PEAK_HBM_GBS,
             "algorithmic_bytes_per_launch": fft_bytes,
         },
@@ -443,12 +476,107 @@ def time_sfno_forward(batch, iters, warmup, dev, compute="fp32"):
     return times[len(times) // 2], times[0], net, x
 
 
+def sfno_kernel_classes(dev, net, iters=10):
+    """Every kernel class of the SFNO-8L forward (batch 1) timed on its own at its in-model shape with HIP events, next to the
+    work the class does per launch and the roofline that bounds it.  Transform stages go through the C ABI on the network's own
+    plans, the 1x1 convolutions through the fused kernels on the network's own weights.  Returns {class: {...}} with calls per
+    forward, so that sum(calls * ms) can be held against the measured forward time."""
+    import torch
+    import makani_amd.pointwise as pw
+    from makani_amd import _lib
+    from makani_amd._lib import lib, check
+
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    C = net.embed_dim
+    out = {}
+
+    def hbm(name, calls, ms, nbytes):
+        out[name] = {"calls": calls, "ms": ms, "bound": "hbm", "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / ms / 1e6,
+                     "frac": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+
+    def mfma(name, calls, ms, flops, nbytes):
+        # bf16 matrix pipe; at these shapes the byte stream is the binding roof when bytes / 8 TB/s exceeds flops / 2.5 PFLOP/s
+        t_hbm, t_pipe = nbytes / (PEAK_HBM_GBS * 1e9), flops / (PEAK_BF16_MFMA_TFLOPS * 1e12)
+        bound = "hbm" if t_hbm >= t_pipe else "mfma"
+        out[name] = {"calls": calls, "ms": ms, "bound": bound, "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
+                     "achieved_GBps": nbytes / ms / 1e6, "achieved_TFLOPs": flops / ms / 1e9,
+                     "frac": max(t_hbm, t_pipe) / (ms * 1e-3)}
+
+    big, small = net.trans_down, net.trans
+    nl = len(net.blocks)
+    for tag, fwd, inv, n_r, n_i in (("721x1440", net.trans_down, net.itrans_up, 1, 2), ("240x480", net.trans, net.itrans, nl - 1, nl)):
+        nlat, nlon, lmax, mmax = fwd.nlat, fwd.nlon, fwd.lmax, fwd.mmax
+        pf, pi = fwd.plan(dev).handle, inv.plan(dev).handle
+        x = torch.randn(C, nlat, nlon, device=dev).to(torch.bfloat16)
+        xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
+        spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
+        fft_bytes = C * nlat * nlon * 2 + C * nlat * mmax * 8
+        T = triangular_count(lmax, mmax)
+        Tp = sum(min(l + 1, mmax) for l in range(lmax))
+        leg_bytes = C * nlat * mmax * 8 + T * nlat * 4 + C * Tp * 8
+        leg_flops = 4.0 * C * nlat * T / 2 * 6          # executed: equator fold, six bf16 products per fp32 product
+        t = event_time_ms(lambda: check(lib.sfno_rfft(pf, P(x), _lib.DTYPE_BF16, P(xm), C, sp), "rfft"), iters, stream)
+        hbm(f"rfft {tag} bf16 in", n_r, t, fft_bytes)
+        t = event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream)
+        mfma(f"legendre analysis {tag}", n_r, t, leg_flops, leg_bytes)
+        t = event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream)
+        mfma(f"legendre synthesis {tag}", n_i, t, leg_flops, leg_bytes)
+        t = event_time_ms(lambda: check(lib.sfno_irfft(pi, P(xm), P(x), _lib.DTYPE_BF16, C, sp), "irfft"), iters, stream)
+        hbm(f"irfft {tag} bf16 out", n_i, t, fft_bytes)
+        if tag == "240x480":
+            from makani_amd.contractions import dhconv_spectral
+            w = net.blocks[1].filter.filter.weight
+            t = event_time_ms(lambda: dhconv_spectral(spec, w, 1, mmax), iters, stream)
+            mfma("dhconv 384x384x240", nl, t, 8.0 * C * C * Tp * 6 / 4 * 2, C * C * lmax * 8 + 2 * C * Tp * 8)
+        del x, xm, spec
+    # 1x1 convolutions of the pointwise tail: (name, module weight, bias, act, addend?, resolution, calls)
+    hw_big, hw_small = net.inp_shape, (net.h, net.w)
+    blk, last = net.blocks[1], net.blocks[-1]
+    convs = [("conv 73->384 +GELU 721x1440", net.encoder.fwd[0], "gelu", False, hw_big, 1),
+             ("conv 384->384 721x1440", net.encoder.fwd[2], None, False, hw_big, 1),
+             ("conv 384->768 +GELU 240x480", blk.mlp.fwd[0], "gelu", False, hw_small, nl - 1),
+             ("conv 768->384 240x480", blk.mlp.fwd[3], None, False, hw_small, nl - 1),
+             ("conv 384->384 +addend 240x480", blk.outer_skip, None, True, hw_small, nl - 1),
+             ("conv 384->768 +GELU 721x1440", last.mlp.fwd[0], "gelu", False, hw_big, 1),
+             ("conv 768->384 721x1440", last.mlp.fwd[3], None, False, hw_big, 1),
+             ("conv 384->384 +addend 721x1440", last.outer_skip, None, True, hw_big, 1),
+             ("conv 384->384 +GELU 721x1440", net.decoder.fwd[0], "gelu", False, hw_big, 1),
+             ("conv 384->73 +addend 721x1440", net.decoder.fwd[2], None, True, hw_big, 1),
+             ("conv 73->73 721x1440", net.residual_transform, None, False, hw_big, 1)]
+    for name, mod, act, add, (h, w_), calls in convs:
+        O, K = mod.weight.shape[0], mod.weight.shape[1]
+        xin = torch.randn(1, K, h, w_, device=dev).to(torch.bfloat16)
+        addend = torch.randn(1, O, h, w_, device=dev).to(torch.bfloat16) if add else None
+        sc = torch.ones(1, O, device=dev) if add else None
+        sh = torch.zeros(1, O, device=dev) if add else None
+        t = event_time_ms(lambda: pw.conv1x1(xin, mod.weight, mod.bias, act, addend, sc, sh), iters, stream)
+        npx = h * w_
+        mfma(name, calls, t, 2.0 * K * O * npx, 2 * npx * (K + O + (O if add else 0)))
+        del xin, addend
+    # instance-norm statistics and the scale/shift/GELU pass
+    for tag, (h, w_), calls in (("240x480", hw_small, nl - 1), ("721x1440", hw_big, 1)):
+        xin = torch.randn(1, C, h, w_, device=dev).to(torch.bfloat16)
+        t = event_time_ms(lambda: pw.instance_norm_coeffs(xin), iters, stream)
+        hbm(f"instance-norm statistics {tag}", calls, t, 2 * C * h * w_)
+        sc, sh = pw.instance_norm_coeffs(xin)
+        t = event_time_ms(lambda: pw.scale_shift_act(xin, sc, sh, "gelu"), iters, stream)
+        hbm(f"scale+shift+GELU {tag}", calls, t, 4 * C * h * w_)
+        del xin
+    return out
+
+
 def bench_sfno8l(args):
     import torch
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    med, best, _, _ = time_sfno_forward(1, max(args.steps, 5), args.warmup, dev, args.compute)
+    med, best, net, xin = time_sfno_forward(1, max(args.steps, 5), args.warmup, dev, args.compute)
+    del xin
+    torch.cuda.empty_cache()
+    with torch.inference_mode():
+        classes = sfno_kernel_classes(dev, net) if args.compute == "fp32" else None
     return {
         "metric": "SFNO-L8 fwd ms/sample", "value": med, "unit": "ms/sample", "n_gpus": 1, "steps": max(args.steps, 5), "warmup": args.warmup,
         "ms_per_step": med, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -457,6 +585,8 @@ def bench_sfno8l(args):
         "config": {"workload": "configs[3]: SFNO-linear 8 layers, embed 384, scale factor 3 (721x1440 -> 240x480), 73 channels, batch 1, "
                                "bf16 autocast forward, random-init weights, N(0,1) inputs"},
         "best_ms": best,
+        "kernel_classes_ms_sum": sum(c["calls"] * c["ms"] for c in classes.values()) if classes else None,
+        "kernel_classes": classes,
     }
 
 
@@ -511,9 +641,15 @@ def main():
         if not args.no_sfno:
             # the second headline figure of the metric, measured in the same run
             torch.cuda.empty_cache()
-            med, best, _, _ = time_sfno_forward(1, 10, 3, torch.device("cuda:0"))
+            med, best, net, xin = time_sfno_forward(1, 10, 3, torch.device("cuda:0"))
+            del xin
+            torch.cuda.empty_cache()
+            with torch.inference_mode():
+                classes = sfno_kernel_classes(torch.device("cuda:0"), net)
             res["sfno_l8_fwd_ms_per_sample"] = {"value": med, "best": best, "batch": 1, "dtype": "bf16 pointwise / f32 spectral",
-                                                "config": "configs[3]: SFNO-linear 8 layers, embed 384, 721x1440, 73 channels, bf16 autocast"}
+                                                "config": "configs[3]: SFNO-linear 8 layers, embed 384, 721x1440, 73 channels, bf16 autocast",
+                                                "kernel_classes_ms_sum": sum(c["calls"] * c["ms"] for c in classes.values()),
+                                                "kernel_classes": classes}
     elif args.workload == "fft2_pair":
         res = bench_fft2_pair(args)
     elif args.workload == "spectral_block":

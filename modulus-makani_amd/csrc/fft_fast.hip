@@ -854,9 +854,11 @@ int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t r
     constexpr int H = 8 / S;                            // batches per tile: a tile owns 8 pairs = one 128-byte line per order
     constexpr int FT = (S * N >= 4096) ? 512 : 256;     // threads per workgroup
     const int ngroups = (ld / 4 + S * H - 1) / (S * H);
-    // two resident workgroups per CU, the same number on every XCD; fewer when an XCD has fewer tiles than that
+    // as many workgroups as stay resident (four wavefronts per SIMD: two workgroups of 512 threads or four of 256 per CU), the
+    // same number on every XCD; fewer when an XCD has fewer tiles than that
+    constexpr int WG_PER_CU = 1024 / FT;
     const int64_t tiles_xcd = (int64_t)((nlat + 7) / 8) * ngroups;
-    const int per_xcd = (int)std::min<int64_t>(tiles_xcd, std::max(1, 2 * p.n_cu / 8));
+    const int per_xcd = (int)std::min<int64_t>(tiles_xcd, std::max(1, WG_PER_CU * p.n_cu / 8));
     dim3 grid((unsigned)(8 * per_xcd));
     if (!inverse) {
         float scale = (float)(kTwoPi / (double)N);
@@ -870,7 +872,7 @@ int go_fast(bool inverse, const FftPlan& p, const void* in, void* out, int64_t r
         const float* xm = reinterpret_cast<const float*>(in);
         const bool small = mmax <= NSMALL * TP;
         const int ng = small ? ngroups : (ld / 4 + S - 1) / S;
-        const int per = (int)std::min<int64_t>((int64_t)((nlat + 7) / 8) * ng, std::max(1, 2 * p.n_cu / 8));
+        const int per = (int)std::min<int64_t>((int64_t)((nlat + 7) / 8) * ng, std::max(1, WG_PER_CU * p.n_cu / 8));
 #define IRFFT_GO(H_, NSWA_, LS_)                                                                                                            \
     hipLaunchKernelGGL((irfft_fast_kernel<N, R0, R1, R2, S, H_, FT, BF16, NSWA_, LS_>), dim3((unsigned)(8 * per)), dim3(FT), 0, s, p.d_tw0, \
                        p.d_tw1, p.d_post, xm, out, rows, nlat, mmax, ld, ng, lat_stats)

@@ -228,7 +228,8 @@ def bench_sht_pair(args):
         # what the matrix pipe executes: half the algorithmic MACs (equator fold), each as six bf16 products (one in bf16 mode)
         executed = leg_flops / 2 * (6 if args.compute == "fp32" else 1)
         roofline = {"kernel": f"legendre_fold_kernel ({dom})", "bound": "hbm", "achieved": hbm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": hbm_gbs / PEAK_HBM_GBS, "traffic": read_traffic(dom, tnote), "algorithmic_bytes_per_launch": leg_bytes,
+                    "frac": hbm_gbs / PEAK_HBM_GBS, "traffic": read_traffic(dom, tnote) if args.compute == "fp32" else None,
+                    "algorithmic_bytes_per_launch": leg_bytes,
                     "avg_launch_ms": stage_ms[dom], "against_fp32_mfma_peak": mfma_view,
                     "executed_on_bf16_pipe": {"flops_per_launch": executed, "achieved_TFLOPs": executed / (stage_ms[dom] * 1e-3) / 1e12,
                                               "peak_TFLOPs": PEAK_BF16_MFMA_TFLOPS, "frac": executed / (stage_ms[dom] * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS},

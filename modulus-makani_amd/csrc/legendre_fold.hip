@@ -1,4 +1,6 @@
-// Equator-folded Legendre contractions on fp32 MFMA (v_mfma_f32_32x32x2_f32), gfx950.
+// Equator-folded Legendre contractions on the matrix cores of gfx950: fp32 results from the bf16 pipe (operands cut
+// exactly into three bf16 planes, six v_mfma_f32_32x32x16_bf16 per K step; the default), the fp32 instruction
+// v_mfma_f32_32x32x2_f32, or plain bf16 operands -- see MODE below.
 //
 //   analysis : spec[m][l][n] = sum_k W[m][l][k] xm[m][k][n]     (RealSHT.forward, Legendre stage)
 //   synthesis: xm[m][k][n]   = sum_l P[m][l][k] spec[m][l][n]   (InverseRealSHT.forward, Legendre stage)

@@ -105,6 +105,19 @@ int sfno_quadrature(int grid, int nlat, double* theta, double* w);
 int sfno_legendre_table(int mmax, int lmax, int nlat, const double* theta, int norm,
                         int inverse, int csphase, double* out);
 
+/* Which part of that table a plan streams.  Towards the poles Pbar_l^m falls off like
+ * sin^m(theta), so the device streams (32-row blocks x K chunks of 16 over the northern
+ * latitudes, per order m and parity p of l + m) leave out the leading chunks of a row block
+ * whose entries are all at most 2^-64 of the largest entry of the order.  Writes the number
+ * of omitted chunks of every row block, in stream order (m, p, row block), to skips (at most
+ * `capacity` values) and returns the number of row blocks, or a negative error code.
+ * analysis != 0: rows are the degrees l = m + p + 2 i, K runs over the latitudes and the
+ * entries carry lat_w[k] (may be null); otherwise rows are the latitudes and K runs over i.
+ * No counterpart in the reference (its tables are dense); host-only, for tests and sizing. */
+int64_t sfno_legendre_stream_skips(int mmax, int lmax, int nlat, const double* theta, const double* lat_w,
+                                   int norm, int inverse, int csphase, int analysis, int32_t* skips,
+                                   int64_t capacity);
+
 /* ---- transform plans --------------------------------------------------------------- */
 
 /* Builds the packed Legendre tables and FFT twiddles on the current HIP device.

@@ -36,7 +36,8 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     LegendreGen gen(p.mmax, p.lmax, p.nlat, theta, p.norm, inverse ? 1 : 0, p.csphase);
     std::vector<float> packed;
     std::vector<int64_t> aoff;
-    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.format, packed, aoff);
+    std::vector<double> kept;          // mean number of K chunks a row block of order m runs through
+    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.format, packed, aoff, &kept);
     // a workgroup covers two 32-row blocks of each parity
     const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
@@ -45,11 +46,10 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
         int nl0 = (p.lmax - m > 0) ? (p.lmax - m + 1) / 2 : 0;
         if (analysis) {
             nrb[m] = (nl0 + PG_ROWS - 1) / PG_ROWS;
-            cost[m] = 1.0;
         } else {
             nrb[m] = (K2 + PG_ROWS - 1) / PG_ROWS;       // orders without any degree still zero-fill their rows
-            cost[m] = 1.0 + (nl0 + PG_KC - 1) / PG_KC;
         }
+        cost[m] = 1.0 + kept[m];
     }
     std::vector<int2> work;
     build_worklist(nrb, cost, work, 2);

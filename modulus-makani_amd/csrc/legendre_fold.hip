@@ -88,11 +88,25 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
 
     const float* xm_m = (ANALYSIS ? a.Q : a.Out) + (int64_t)m * nlat * ld;     // Fourier panel of order m
     const float* sp_m = (ANALYSIS ? a.Out : a.Q) + (int64_t)m * lmax * ld;     // spectral panel of order m
-    // wavefronts without a row block read the head of the table (always at least nc blocks long) and discard it
+    // wavefronts without a row block read the head of the table and discard it
     // 16 bytes per lane: fp32 blocks are two such pieces per chunk (128 per block), bf16 blocks one (64 per block)
     constexpr int NA = MODE == LF_BF16 ? 1 : MODE == LF_SPLIT ? 3 : 2;     // 16-byte pieces per lane and block
     constexpr int APB = 64 * NA;
-    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((active ? a.a_off[2 * m + par] + (int64_t)rb * nc : (int64_t)0) * APB + lane);
+    // Index entry of a row block: first block of its stream | leading chunks left out << 48 (their entries are negligible:
+    // towards the poles the table falls off like sin^m(theta)).  The K loop of the workgroup starts at the smallest such
+    // count of its (up to) four row blocks; a wavefront joins in at its own.
+    auto entry_of = [&](int p_, int rb_) {
+        const int nr = ANALYSIS ? (p_ ? nl1 : nl0) : K2;
+        // an order without degrees (synthesis with mmax > lmax: nc = 0) has no entries; its rows are zero-filled below
+        return (nc > 0 && rb_ * PG_ROWS < nr) ? a.a_off[a.a_off[2 * m + p_] + rb_] : (int64_t)nc << 48;
+    };
+    int cstart = nc;
+#pragma unroll
+    for (int s_ = 0; s_ < 4; ++s_) cstart = min(cstart, (int)(entry_of(s_ >> 1, wi.y + (s_ & 1)) >> 48));
+    const int64_t my_entry = entry_of(par, rb);
+    cstart = max(cstart, 0);
+    const int c0w = min(max((int)(my_entry >> 48), 0), nc);   // nc for a wavefront without a row block or with nothing but negligible entries
+    const float4* ap = reinterpret_cast<const float4*>(a.A) + ((c0w < nc ? my_entry & (((int64_t)1 << 48) - 1) : (int64_t)0) * APB + lane);
 
     floatx16 acc[NT];
 #pragma unroll
@@ -213,7 +227,7 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
     const f4* apv = reinterpret_cast<const f4*>(ap);
     auto a_load = [&](int c, f4 (&ar)[NA]) {
 #pragma unroll
-        for (int p = 0; p < NA; ++p) ar[p] = apv[(int64_t)c * APB + 64 * p];
+        for (int p = 0; p < NA; ++p) ar[p] = apv[(int64_t)max(c - c0w, 0) * APB + 64 * p];
     };
 
     // Software pipeline, one chunk deep: the loads of chunk c+1 (raw panel rows and table
@@ -221,14 +235,14 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
     // The explicit wait for all of them at the end of the iteration keeps the wait-count
     // bookkeeping of the next iteration's MFMA block empty.
     f4 acur[NA], anext[NA];
-    if (nc > 0) {
-        q_load(0);
-        a_load(0, acur);
-        q_store(0, 0);
+    if (cstart < nc) {
+        q_load(cstart);
+        a_load(cstart, acur);
+        q_store(cstart & 1, cstart);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): the first table fragments too
     __syncthreads();
-    for (int c = 0; c < nc; ++c) {
+    for (int c = cstart; c < nc; ++c) {
         const int buf = c & 1;
         const bool more = c + 1 < nc;
         if (more) {
@@ -236,7 +250,7 @@ __global__ __launch_bounds__(256, lf_occupancy(NT, MODE)) void legendre_fold_ker
             a_load(c + 1, anext);
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (active) compute(buf, acur);
+        if (c >= c0w) compute(buf, acur);
         __builtin_amdgcn_sched_barrier(0);
         if (more) q_store(buf ^ 1, c + 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): everything issued above has landed

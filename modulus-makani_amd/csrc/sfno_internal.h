@@ -23,7 +23,7 @@ constexpr int PG_WAVES = 4;        // wavefronts (= row blocks) per workgroup
 
 struct PgemmTable {
     float* d_A = nullptr;          // packed stream
-    int64_t* d_aoff = nullptr;     // [nbatch] first block of each batch
+    int64_t* d_aoff = nullptr;     // index of the stream, see pack_legendre_fold
     int2* d_work = nullptr;        // [n_work] {batch, first row block} per workgroup, -1 = idle
     int n_work = 0;                // multiple of 8 (one queue per XCD, interleaved)
     int64_t n_blocks = 0;
@@ -118,8 +118,11 @@ void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost
 enum { PG_FORMAT_FP32 = 0, PG_FORMAT_BF16 = 1, PG_FORMAT_SPLIT = 2 };
 inline int pg_block_floats(int format) { return format == PG_FORMAT_BF16 ? 256 : format == PG_FORMAT_SPLIT ? 768 : 512; }
 // value = P * lat_w[k] * order_scale[m]; a null pointer stands for all ones
+// aoff: [2 m + p] -> position in aoff of the stream's first row-block entry; entry of row block rb (at that position + rb) =
+// first block of the row block | (number of leading K chunks left out as negligible << 48); chunks_per_rb (optional): mean
+// number of kept chunks per row block of every order (work-list cost)
 void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
-                        std::vector<float>& packed, std::vector<int64_t>& aoff);
+                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb = nullptr);
 int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------

@@ -167,23 +167,18 @@ static void parallel_for(int n, F f) {
     for (auto& x : th) x.join();
 }
 
-// Packs P (rows x K, accessed through get(row,k)) into the fragment stream described in
-// sfno_internal.h.  dst has nrb*nc blocks.
+// One 32 x 16 block (row block rb, K chunk c) of P (rows x K, accessed through get(row, k)) as the fragment stream
+// described in sfno_internal.h wants it.
 template <class G>
-static void pack_blocks(float* dst, int rows, int K, G get) {
-    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
-    for (int rb = 0; rb < nrb; ++rb)
-        for (int c = 0; c < nc; ++c) {
-            float* blk = dst + ((size_t)rb * nc + c) * PG_BLOCK_FLOATS;
-            for (int h = 0; h < 2; ++h)
-                for (int j = 0; j < 64; ++j)
-                    for (int s = 0; s < 4; ++s) {
-                        int row = PG_ROWS * rb + (j & 31);
-                        int k = PG_KC * c + 8 * h + 2 * s + (j >> 5);
-                        float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
-                        blk[(h * 64 + j) * 4 + s] = v;
-                    }
-        }
+static void pack_block(float* blk, int rb, int c, int rows, int K, G get) {
+    for (int h = 0; h < 2; ++h)
+        for (int j = 0; j < 64; ++j)
+            for (int s = 0; s < 4; ++s) {
+                int row = PG_ROWS * rb + (j & 31);
+                int k = PG_KC * c + 8 * h + 2 * s + (j >> 5);
+                float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
+                blk[(h * 64 + j) * 4 + s] = v;
+            }
 }
 
 // Folded tables: the grids are symmetric about the equator and Pbar_l^m(pi - theta) =
@@ -203,93 +198,139 @@ static unsigned short bf16_rne(double v) {
     return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 
-// bf16 flavour of pack_blocks: block = 64 lanes x 8 bf16; lane j holds P[32 rb + (j & 31)][16 c + 8 (j >> 5) + e], e = 0..7
+// bf16 flavour: block = 64 lanes x 8 bf16; lane j holds P[32 rb + (j & 31)][16 c + 8 (j >> 5) + e], e = 0..7
 template <class G>
-static void pack_blocks_bf16(unsigned short* dst, int rows, int K, G get) {
-    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
-    for (int rb = 0; rb < nrb; ++rb)
-        for (int c = 0; c < nc; ++c) {
-            unsigned short* blk = dst + ((size_t)rb * nc + c) * PG_BLOCK_FLOATS;
-            for (int j = 0; j < 64; ++j)
-                for (int e = 0; e < 8; ++e) {
-                    int row = PG_ROWS * rb + (j & 31);
-                    int k = PG_KC * c + 8 * (j >> 5) + e;
-                    blk[j * 8 + e] = (row < rows && k < K) ? bf16_rne(get(row, k)) : (unsigned short)0;
-                }
+static void pack_block_bf16(unsigned short* blk, int rb, int c, int rows, int K, G get) {
+    for (int j = 0; j < 64; ++j)
+        for (int e = 0; e < 8; ++e) {
+            int row = PG_ROWS * rb + (j & 31);
+            int k = PG_KC * c + 8 * (j >> 5) + e;
+            blk[j * 8 + e] = (row < rows && k < K) ? bf16_rne(get(row, k)) : (unsigned short)0;
         }
 }
 
-// three-plane flavour: block = 3 planes x 64 lanes x 8 bf16, same (lane, e) -> (row, k) map as pack_blocks_bf16; the planes
+// three-plane flavour: block = 3 planes x 64 lanes x 8 bf16, same (lane, e) -> (row, k) map as the bf16 flavour; the planes
 // hold the fp32 value cut into its upper, middle and lower 8 significant bits (truncation, so the sum is exact)
 template <class G>
-static void pack_blocks_split(unsigned short* dst, int rows, int K, G get) {
-    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
-    for (int rb = 0; rb < nrb; ++rb)
-        for (int c = 0; c < nc; ++c) {
-            unsigned short* blk = dst + ((size_t)rb * nc + c) * 1536;
-            for (int j = 0; j < 64; ++j)
-                for (int e = 0; e < 8; ++e) {
-                    int row = PG_ROWS * rb + (j & 31);
-                    int k = PG_KC * c + 8 * (j >> 5) + e;
-                    float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
-                    for (int pl = 0; pl < 3; ++pl) {
-                        uint32_t u;
-                        std::memcpy(&u, &v, 4);
-                        u &= 0xffff0000u;
-                        float t;
-                        std::memcpy(&t, &u, 4);
-                        blk[(pl * 64 + j) * 8 + e] = (unsigned short)(u >> 16);
-                        v -= t;
-                    }
-                }
+static void pack_block_split(unsigned short* blk, int rb, int c, int rows, int K, G get) {
+    for (int j = 0; j < 64; ++j)
+        for (int e = 0; e < 8; ++e) {
+            int row = PG_ROWS * rb + (j & 31);
+            int k = PG_KC * c + 8 * (j >> 5) + e;
+            float v = (row < rows && k < K) ? (float)get(row, k) : 0.0f;
+            for (int pl = 0; pl < 3; ++pl) {
+                uint32_t u;
+                std::memcpy(&u, &v, 4);
+                u &= 0xffff0000u;
+                float t;
+                std::memcpy(&t, &u, 4);
+                blk[(pl * 64 + j) * 8 + e] = (unsigned short)(u >> 16);
+                v -= t;
+            }
         }
+}
+
+// Stream of one (order, parity): for every row block the chunks from its first non-negligible one on.  Towards the
+// poles Pbar_l^m falls off like sin^m(theta) (and faster below the turning latitude sin(theta) = m / l): the leading
+// chunks of a row block whose entries are all at most `thr` in magnitude are left out -- `skip[rb]` of them, the kernel
+// starts that row block's K loop there.  With thr = 2^-64 of the largest entry of the order the omitted terms are 2^-40
+// of one fp32 rounding of the result.
+template <class G>
+static void pack_stream(std::vector<float>& out, std::vector<int>& skip, int rows, int K, int format, double thr, G get) {
+    const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
+    const size_t bf = (size_t)pg_block_floats(format);
+    for (int rb = 0; rb < nrb; ++rb) {
+        int c0 = 0;
+        for (; c0 < nc; ++c0) {
+            bool negligible = true;
+            for (int row = PG_ROWS * rb; row < std::min(rows, PG_ROWS * (rb + 1)) && negligible; ++row)
+                for (int k = PG_KC * c0; k < std::min(K, PG_KC * (c0 + 1)); ++k)
+                    if (std::fabs(get(row, k)) > thr) {
+                        negligible = false;
+                        break;
+                    }
+            if (!negligible) break;
+        }
+        skip.push_back(c0);
+        const size_t at = out.size();
+        out.resize(at + (size_t)(nc - c0) * bf, 0.0f);
+        for (int c = c0; c < nc; ++c) {
+            float* blk = out.data() + at + (size_t)(c - c0) * bf;
+            if (format == PG_FORMAT_BF16) pack_block_bf16(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get);
+            else if (format == PG_FORMAT_SPLIT) pack_block_split(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get);
+            else pack_block(blk, rb, c, rows, K, get);
+        }
+    }
 }
 
 void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
-                        std::vector<float>& packed, std::vector<int64_t>& aoff) {
+                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb) {
     const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
     const int K2 = (nlat + 1) / 2;
     auto nl_p = [&](int m, int p) { return (lmax - m - p > 0) ? (lmax - m - p + 1) / 2 : 0; };
-    aoff.assign((size_t)2 * mmax, 0);
-    int64_t tot = 0;
-    for (int m = 0; m < mmax; ++m)
-        for (int p = 0; p < 2; ++p) {
-            aoff[2 * m + p] = tot;
-            int64_t nrb = analysis ? (nl_p(m, p) + PG_ROWS - 1) / PG_ROWS : (K2 + PG_ROWS - 1) / PG_ROWS;
-            int64_t nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl_p(m, 0) + PG_KC - 1) / PG_KC;
-            tot += nrb * nc;
-        }
-    const size_t blk_floats = (size_t)pg_block_floats(format);
-    packed.assign((size_t)tot * blk_floats, 0.0f);
-    float* base = packed.data();
-    parallel_for(mmax, [&, base](int m) {
+    // per (order, parity): the packed blocks and the number of skipped leading chunks of every row block
+    std::vector<std::vector<float>> part((size_t)2 * mmax);
+    std::vector<std::vector<int>> skip((size_t)2 * mmax);
+    parallel_for(mmax, [&](int m) {
         int nl = lmax - m;
-        if (nl <= 0) return;
+        if (nl <= 0) {
+            // no degrees: the synthesis still has its row blocks (they produce zeros), each with an empty K loop
+            if (!analysis)
+                for (int p = 0; p < 2; ++p) skip[2 * m + p].assign((size_t)(K2 + PG_ROWS - 1) / PG_ROWS, 0);
+            return;
+        }
         std::vector<double> rows((size_t)nl * nlat);
         g.rows_for_m(m, rows.data());
         const double* r = rows.data();
+        const double sc = order_scale ? order_scale[m] : 1.0;
+        auto lw = [=](int k) { return lat_w ? lat_w[k] * sc : sc; };
+        double vmax = 0.0;
+        for (int i = 0; i < nl; ++i)
+            for (int k = 0; k < K2; ++k) vmax = std::max(vmax, std::fabs(r[(size_t)i * nlat + k] * lw(k)));
+        const double thr = std::ldexp(vmax, -64);
         for (int p = 0; p < 2; ++p) {
             const int np = nl_p(m, p);
-            float* dst = base + (size_t)aoff[2 * m + p] * blk_floats;
             // K extent of the synthesis padded to the even-parity chunk count so that both parities run the same loop
             const int kpad = nl_p(m, 0);
-            const double sc = order_scale ? order_scale[m] : 1.0;
-            auto lw = [=](int k) { return lat_w ? lat_w[k] * sc : sc; };
             auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * lw(k); };
             auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] * lw(row) : 0.0; };
-            unsigned short* d16 = reinterpret_cast<unsigned short*>(dst);
-            if (format == PG_FORMAT_BF16) {
-                if (analysis) pack_blocks_bf16(d16, np, K2, wa);
-                else pack_blocks_bf16(d16, K2, kpad, ws);
-            } else if (format == PG_FORMAT_SPLIT) {
-                if (analysis) pack_blocks_split(d16, np, K2, wa);
-                else pack_blocks_split(d16, K2, kpad, ws);
-            } else {
-                if (analysis) pack_blocks(dst, np, K2, wa);
-                else pack_blocks(dst, K2, kpad, ws);
-            }
+            if (analysis) pack_stream(part[2 * m + p], skip[2 * m + p], np, K2, format, thr, wa);
+            else pack_stream(part[2 * m + p], skip[2 * m + p], K2, kpad, format, thr, ws);
         }
     });
+    // index: aoff[2 m + p] = position (in aoff) of the first row-block entry of that stream; an entry is
+    // (first block of the row block in the stream) | (skipped chunks << 48)
+    const size_t blk_floats = (size_t)pg_block_floats(format);
+    size_t nent = 0, nfl = 0;
+    for (size_t b = 0; b < part.size(); ++b) {
+        nent += skip[b].size();
+        nfl += part[b].size();
+    }
+    aoff.assign((size_t)2 * mmax + nent, 0);
+    packed.resize(nfl);
+    if (chunks_per_rb) chunks_per_rb->assign(mmax, 0.0);
+    size_t ent = (size_t)2 * mmax, blk = 0, fl = 0;
+    for (int m = 0; m < mmax; ++m) {
+        double kept = 0.0;
+        size_t nrb_m = 0;
+        for (int p = 0; p < 2; ++p) {
+            const size_t b = (size_t)2 * m + p;
+            aoff[b] = (int64_t)ent;
+            const int64_t nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl_p(m, 0) + PG_KC - 1) / PG_KC;
+            for (int c0 : skip[b]) {
+                aoff[ent++] = (int64_t)blk | ((int64_t)c0 << 48);
+                blk += (size_t)(nc - c0);
+                kept += (double)(nc - c0);
+                ++nrb_m;
+            }
+            if (!part[b].empty()) std::memcpy(packed.data() + fl, part[b].data(), sizeof(float) * part[b].size());
+            fl += part[b].size();
+            std::vector<float>().swap(part[b]);
+        }
+        if (chunks_per_rb && nrb_m) (*chunks_per_rb)[m] = kept / (double)nrb_m;
+    }
+    // the kernel's wavefronts without a row block read (and discard) the head of the stream: keep it at least one block long
+    if (packed.size() < blk_floats) packed.resize(blk_floats, 0.0f);
 }
 
 void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost, std::vector<int2>& work, int rb_step) {
@@ -337,4 +378,17 @@ extern "C" int sfno_legendre_table(int mmax, int lmax, int nlat, const double* t
         std::memcpy(out + ((size_t)m * lmax + m) * nlat, rows.data(), sizeof(double) * (size_t)(lmax - m) * nlat);
     }
     return SFNO_OK;
+}
+
+extern "C" int64_t sfno_legendre_stream_skips(int mmax, int lmax, int nlat, const double* theta, const double* lat_w, int norm, int inverse,
+                                              int csphase, int analysis, int32_t* skips, int64_t capacity) {
+    if (mmax < 1 || lmax < 1 || nlat < 1 || !theta || capacity < 0 || (capacity > 0 && !skips)) return SFNO_EINVAL;
+    if (norm < 0 || norm > 2) return SFNO_EINVAL;
+    sfno::LegendreGen g(mmax, lmax, nlat, theta, norm, inverse, csphase);
+    std::vector<float> packed;
+    std::vector<int64_t> aoff;
+    sfno::pack_legendre_fold(g, lat_w, nullptr, analysis != 0, sfno::PG_FORMAT_BF16, packed, aoff);
+    const int64_t n = (int64_t)aoff.size() - 2 * (int64_t)mmax;
+    for (int64_t i = 0; i < n && i < capacity; ++i) skips[i] = (int32_t)(aoff[(size_t)(2 * mmax + i)] >> 48);
+    return n;
 }

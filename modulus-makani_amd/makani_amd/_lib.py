@@ -37,6 +37,7 @@ def _load():
         "sfno_version": (i32, []),
         "sfno_quadrature": (i32, [i32, i32, dp, dp]),
         "sfno_legendre_table": (i32, [i32, i32, i32, dp, i32, i32, i32, dp]),
+        "sfno_legendre_stream_skips": (i64, [i32, i32, i32, dp, dp, i32, i32, i32, i32, c.POINTER(c.c_int32), i64]),
         "sfno_sht_plan_create": (i32, [i32, i32, i32, i32, i32, i32, i32, i32, i32, c.POINTER(vp)]),
         "sfno_sht_plan_destroy": (i32, [vp]),
         "sfno_spectral_ld": (i64, [i64]),

@@ -99,3 +99,62 @@ def test_module_attributes_and_errors(lib_built):
     assert ma.SpectralConv(s, ma.InverseRealSHT(16, 32, lmax=32, mmax=33, grid="legendre-gauss"), 4, 6, operator_type="dhconv").scale_residual
     with pytest.raises(ValueError):
         ma.SpectralConv(s, ma.InverseRealSHT(32, 64, grid="legendre-gauss"), 4, 6, operator_type="bogus")
+
+
+@pytest.mark.parametrize("nlat,lmax,mmax,grid", [(241, 241, 241, "legendre-gauss"), (361, 240, 241, "equiangular"), (32, 32, 33, "equiangular")])
+@pytest.mark.parametrize("analysis", [True, False])
+def test_stream_leaves_out_only_negligible_polar_chunks(lib_built, nlat, lmax, mmax, grid, analysis):
+    """The device streams of the Legendre tables omit the leading K chunks of a 32-row block whose entries are all at most
+    2^-64 of the largest entry of the order.  Checked against the oracle's float64 table: every omitted entry is that small, the
+    first kept chunk holds a larger one (nothing more could have been dropped at this threshold), the index covers every row block,
+    and at sizes where sin^m(theta) matters a noticeable share of the table is indeed left out."""
+    import ctypes
+
+    import makani_amd._lib as L
+
+    theta, w = grid_nodes(nlat, grid)
+    ref = legpoly(mmax, lmax, theta, "ortho", not analysis, True)          # [m][l][k]
+    if analysis:
+        ref = ref * w[None, None, :]
+    K2 = (nlat + 1) // 2
+    dp = ctypes.POINTER(ctypes.c_double)
+    th = np.ascontiguousarray(theta, dtype=np.float64)
+    lw = np.ascontiguousarray(w, dtype=np.float64)
+    args = (mmax, lmax, nlat, th.ctypes.data_as(dp), lw.ctypes.data_as(dp) if analysis else None, 0, 0 if analysis else 1, 1, 1 if analysis else 0)
+    n = L.lib.sfno_legendre_stream_skips(*args, None, 0)
+    assert n > 0
+    skips = np.zeros(n, dtype=np.int32)
+    assert L.lib.sfno_legendre_stream_skips(*args, skips.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), n) == n
+    pos, dense, kept = 0, 0, 0
+    for m in range(mmax):
+        a = np.abs(ref[m, :, :K2])
+        thr = a.max() * 2.0 ** -64
+        for p in (0, 1):
+            rows_l = np.arange(m + p, lmax, 2)
+            np0 = len(np.arange(m, lmax, 2))
+            if analysis:
+                blk = a[rows_l]                                            # rows = degrees, K = latitudes
+                nc = (K2 + 15) // 16
+            else:
+                blk = np.zeros((K2, np0))                                  # rows = latitudes, K = degrees (padded to parity 0)
+                blk[:, :len(rows_l)] = a[rows_l].T
+                nc = (np0 + 15) // 16
+                if m >= lmax:
+                    blk = np.zeros((K2, 0))
+            nrb = (blk.shape[0] + 31) // 32
+            for rb in range(nrb):
+                c0 = int(skips[pos])
+                pos += 1
+                assert 0 <= c0 <= nc
+                sub = blk[32 * rb:32 * rb + 32]
+                if c0 > 0:
+                    assert sub[:, :16 * c0].max(initial=0.0) <= thr * (1 + 1e-9), (m, p, rb)
+                if c0 < nc:
+                    first = sub[:, 16 * c0:16 * c0 + 16].max(initial=0.0)
+                    assert first > thr * (1 - 1e-9), (m, p, rb, c0)
+                dense += nc
+                kept += nc - c0
+    assert pos == n
+    if nlat >= 241:
+        assert kept < 0.95 * dense
+    print(f"{grid} {nlat} lmax {lmax} mmax {mmax} {'analysis' if analysis else 'synthesis'}: {kept} of {dense} blocks kept")

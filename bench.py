@@ -536,7 +536,8 @@ def sfno_kernel_classes(dev, net, iters=10):
     hw_big, hw_small = net.inp_shape, (net.h, net.w)
     blk, last = net.blocks[1], net.blocks[-1]
     convs = [("conv 73->384 +GELU 721x1440", net.encoder.fwd[0], "gelu", False, hw_big, 1),
-             ("conv 384->384 721x1440", net.encoder.fwd[2], None, False, hw_big, 1),
+             # the encoder's last convolution runs only where the network does not fold it into the first block's spectral weight
+             ("conv 384->384 721x1440", net.encoder.fwd[2], None, False, hw_big, 0 if net._encoder_fold() is not None else 1),
              ("conv 384->768 +GELU 240x480", blk.mlp.fwd[0], "gelu", False, hw_small, nl - 1),
              ("conv 768->384 240x480", blk.mlp.fwd[3], None, False, hw_small, nl - 1),
              ("conv 384->384 +addend 240x480", blk.outer_skip, None, True, hw_small, nl - 1),

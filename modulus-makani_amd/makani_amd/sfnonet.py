@@ -19,6 +19,7 @@ from . import pointwise as pw
 from .sht import RealSHT, InverseRealSHT
 from .layers import RealFFT2, InverseRealFFT2
 from .spectral_convolution import SpectralConv
+from .contractions import dhconv_spectral
 
 _ACTIVATIONS = {"relu": nn.ReLU, "gelu": nn.GELU, "silu": nn.SiLU}
 
@@ -189,7 +190,7 @@ class FourierNeuralOperatorBlock(nn.Module):
             return False
         return hasattr(self, "outer_skip") and _is_conv1x1(self.outer_skip) and self.outer_skip.bias is None
 
-    def _forward_fused(self, x, residual, lat_stats=None):
+    def _forward_fused(self, x, residual, lat_stats=None, skip_weight=None):
         """norm0 -> GELU -> MLP -> norm1 -> + outer_skip(residual) in five kernels: row statistics (or, for norm0, the
         per-latitude moments the inverse transform delivered with x), scale/shift + GELU, two 1x1 convolutions with bias
         (+ GELU) epilogues, row statistics, and the skip convolution whose epilogue adds the normalised MLP output."""
@@ -204,7 +205,9 @@ class FourierNeuralOperatorBlock(nn.Module):
         x = pw.scale_shift_act(x, sc, sh, "gelu")
         x = _run_chain(_fused_chain(self.mlp.fwd), x)
         sc, sh = _norm_coeffs(self.norm1, x)
-        return pw.conv1x1(residual, self.outer_skip.weight, None, None, x, sc, sh)
+        # skip_weight: the skip convolution composed with a linear map the caller pulled out of `residual` (see the network's
+        # _encoder_fold)
+        return pw.conv1x1(residual, self.outer_skip.weight if skip_weight is None else skip_weight, None, None, x, sc, sh)
 
     def forward(self, x):
         # on the fused inference path the inverse transform hands over the moments norm0 needs together with its output
@@ -239,8 +242,12 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                  encoder_layers=1, pos_embed="none", pos_drop_rate=0.0, path_drop_rate=0.0, mlp_drop_rate=0.0,
                  normalization_layer="instance_norm", max_modes=None, hard_thresholding_fraction=1.0, big_skip=True, rank=1.0,
                  factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0,
-                 spectral_compute="fp32", fused_pointwise=True, **kwargs):
+                 spectral_compute="fp32", fused_pointwise=True, fold_encoder=True, **kwargs):
         super().__init__()
+        # fold_encoder (not a Makani option): on the fused inference path the encoder's last (linear) convolution is applied in
+        # spectral space, inside the first block's weights, instead of at full resolution; see _encoder_fold
+        self.fold_encoder = fold_encoder
+        self._fold_cache = None
         # fused_pointwise (not a Makani option): under torch.no_grad() / inference_mode() with bf16 autocast the 1x1 convolutions,
         # instance norms and GELUs run on the fused HIP kernels (weights rounded to bf16 once, fp32 accumulation, one rounding per
         # layer, norm0 statistics from the unrounded field).  A forward that records gradients always runs the PyTorch modules, so
@@ -340,6 +347,56 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                 x = blk(x)
         return x
 
+    # The encoder ends in a bias-free 1x1 convolution W2 (layers.py:129-131) and the first block starts with a transform to a
+    # different grid, so the encoder's output x = W2 h is used by nothing but that transform (the block takes its residual from
+    # the coefficients, spectral_convolution.py:132-134).  Channel mixing commutes with the transforms: SHT(W2 h) = W2 SHT(h).  On
+    # the fused inference path the convolution at full resolution is therefore not run at all: the transform takes h, W2 goes
+    # into the block's spectral weight (w'[j, o, l] = sum_i W2[i, j] w[i, o, l], computed once per weight update) and into the
+    # skip convolution of the residual (W_skip W2).  W2 enters with its bf16-rounded values, as autocast would use it; what
+    # differs from the layer-by-layer evaluation is one bf16 rounding of the 384-channel field that is no longer made.
+    def _encoder_fold(self):
+        """(encoder steps without the last convolution, folded spectral weight, folded skip weight), or None where the
+        shortcut does not apply."""
+        if not getattr(self, "fold_encoder", True) or self.repeat_layers != 1 or len(self.blocks) == 0:
+            return None
+        enc = _fused_chain(self.encoder.fwd)
+        blk = self.blocks[0]
+        conv = blk.filter.filter
+        if enc is None or len(enc) < 2 or enc[-1][1] is not None or enc[-1][0].bias is not None:
+            return None
+        if not (isinstance(blk, FourierNeuralOperatorBlock) and blk._fusable() and getattr(blk, "fused_pointwise", True)):
+            return None
+        if not (conv._fused and conv.scale_residual and not hasattr(conv, "bias") and conv.in_channels == enc[-1][0].out_channels):
+            return None
+        w2, w0, ws = enc[-1][0].weight, conv.weight, blk.outer_skip.weight
+        stamp = tuple((t.data_ptr(), t._version) for t in (w2, w0, ws))
+        cached = getattr(self, "_fold_cache", None)
+        if cached is None or cached[0] != stamp:
+            # (ordinary tensors, also when called under inference_mode: the packed-operand caches read version counters)
+            with torch.inference_mode(False), torch.no_grad():
+                w2b = w2.detach().reshape(w2.shape[0], w2.shape[1]).to(torch.bfloat16).float()        # [i, j]
+                wf = torch.einsum("ij,iol->jol", w2b.to(torch.complex64), w0.detach()).contiguous()
+                wsb = ws.detach().reshape(ws.shape[0], ws.shape[1]).to(torch.bfloat16).float()
+                wsk = (wsb @ w2b).reshape(ws.shape[0], w2.shape[1], 1, 1).contiguous()
+            cached = (stamp, wf, wsk)
+            self._fold_cache = cached
+        return enc[:-1], cached[1], cached[2]
+
+    def clear_fold_cache(self):
+        """Forgets the folded weights (they follow in-place updates of their three parameters through the version counters;
+        call this after writing one of them through ``.data``)."""
+        self._fold_cache = None
+
+    def _block0_folded(self, h, wf, wsk):
+        blk = self.blocks[0]
+        conv = blk.filter.filter
+        B = h.shape[0]
+        spec = conv.forward_transform.analysis(h)
+        residual = conv.inverse_transform.synthesis(spec, (B, h.shape[1]), dtype=torch.bfloat16)
+        spec = dhconv_spectral(spec, wf, B, conv.modes_lon, triangular=conv._triangular, compute=conv.compute)
+        x, stats = conv.inverse_transform.synthesis_with_lat_stats(spec, (B, conv.out_channels), dtype=torch.bfloat16)
+        return blk._forward_fused(x.contiguous(), residual.contiguous(), stats, skip_weight=wsk)
+
     def _forward_fused(self, x):
         """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""
         enc, dec = _fused_chain(self.encoder.fwd), _fused_chain(self.decoder.fwd)
@@ -350,8 +407,14 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
             else:
                 residual = xb
             residual = pw.conv1x1(residual, self.residual_transform.weight)
-        x = _run_chain(enc, xb)
-        x = self._forward_features(x)
+        fold = self._encoder_fold()
+        if fold is not None:
+            x = self._block0_folded(_run_chain(fold[0], xb), fold[1], fold[2])
+            for blk in self.blocks[1:]:
+                x = blk(x)
+        else:
+            x = _run_chain(enc, xb)
+            x = self._forward_features(x)
         return _run_chain(dec, x.to(torch.bfloat16).contiguous(), residual if self.big_skip else None)
 
     def _fusable(self, x):

@@ -68,6 +68,8 @@ def test_sfno8l_every_spectral_block_matches_oracle(lib_built, net8):
     print("case configs[3]: SFNO-8L 721x1440 embed 384, bf16 autocast, per-block SpectralConv vs float64 oracle", flush=True)
     taps = {}
     hooks = []
+    # layer by layer: with the encoder's last convolution folded into block 0 that block's SpectralConv is not called as a module
+    net.fold_encoder = False
     for i, blk in enumerate(net.blocks):
         def hook(mod, args, out, i=i):
             taps[i] = (args[0].detach(), out[0].detach(), out[1].detach())
@@ -75,6 +77,7 @@ def test_sfno8l_every_spectral_block_matches_oracle(lib_built, net8):
     try:
         y = _run(net, x.cuda(), True)
     finally:
+        net.fold_encoder = True
         for h in hooks:
             h.remove()
     torch.cuda.synchronize()
@@ -112,6 +115,9 @@ def test_sfno8l_output_against_float64_oracle_model(lib_built, net8):
     net, x = net8
     print("case configs[3]: SFNO-8L network output, fused kernels and PyTorch bf16 modules vs the float64 oracle model", flush=True)
     y_fused = _run(net, x.cuda(), True).float().cpu().numpy()
+    net.fold_encoder = False
+    y_layers = _run(net, x.cuda(), True).float().cpu().numpy()
+    net.fold_encoder = True
     y_mod = _run(net, x.cuda(), False).float().cpu().numpy()
     torch.cuda.empty_cache()
     t0 = time.time()
@@ -123,6 +129,10 @@ def test_sfno8l_output_against_float64_oracle_model(lib_built, net8):
     # eight bf16 layers deep, both executions carry the rounding of every layer's output; the HIP one must not carry more
     assert e_fused < 3e-2 and e_fused < 1.2 * e_mod
     assert rel_l2(y_fused, y_mod) < e_fused + e_mod
+    # the encoder's last convolution applied in spectral space (fold_encoder) against the same kernels layer by layer
+    e_layers = rel_l2(y_layers, ref)
+    print(f"  layer by layer {e_layers:.3e}, folded vs layer by layer {rel_l2(y_fused, y_layers):.3e}", flush=True)
+    assert e_fused < 1.1 * e_layers and rel_l2(y_fused, y_layers) < e_fused + e_layers
 
 
 def test_rollout_batch4(lib_built, net8):

@@ -200,3 +200,52 @@ def test_fused_pointwise_switch(lib_built):
     assert torch.equal(y_off, y_on_off)
     assert not torch.equal(y_off, y_on)
     assert rel_l2(y_on.float().cpu().numpy(), y_off.float().cpu().numpy()) < 3e-2
+
+
+def test_encoder_fold_matches_layer_by_layer(lib_built):
+    """fold_encoder: the encoder's last (linear, bias-free) 1x1 convolution is applied in spectral space, inside block 0's
+    weights and skip convolution, instead of at full resolution (channel mixing commutes with the transforms).  Same network,
+    folded against layer by layer, both through the float64 oracle model: the folded run must not be further from it, the
+    two must agree within the sum of their distances, the shortcut must really be taken where it applies (grids differ
+    between encoder and block 0) and not where block 0 runs more than once."""
+    case = dict(inp_shape=(92, 180), out_shape=(92, 180), inp_chans=5, out_chans=5, scale_factor=3, embed_dim=48, num_layers=3)
+    print(f"case sfno encoder fold {case}", flush=True)
+    net = build(**case).cuda().eval()
+    g = torch.Generator().manual_seed(11)
+    with torch.no_grad():
+        for n, p in net.named_parameters():
+            if "norm" in n or n.endswith(".bias"):
+                p.add_(0.3 * torch.randn(p.shape, generator=g).to(p.device))
+    x = torch.randn(2, 5, 92, 180, generator=torch.Generator().manual_seed(7))
+
+    def run(fold):
+        net.fold_encoder = fold
+        net.clear_fold_cache()
+        with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+            y = net(x.cuda())
+        return y, net._fold_cache is not None
+
+    (y_fold, taken), (y_layers, taken_off) = run(True), run(False)
+    assert taken and not taken_off
+    ref64 = SfnoOracle((92, 180), (92, 180), 3, 3).forward(net.state_dict(), x).numpy()
+    e_fold = rel_l2(y_fold.float().cpu().double().numpy(), ref64)
+    e_layers = rel_l2(y_layers.float().cpu().double().numpy(), ref64)
+    d = rel_l2(y_fold.float().cpu().numpy(), y_layers.float().cpu().numpy())
+    print(f"folded {e_fold:.3e}  layer by layer {e_layers:.3e}  between them {d:.3e}", flush=True)
+    assert e_fold < 2e-2 and e_fold < 1.1 * e_layers and d < e_fold + e_layers
+    # a weight update is followed: the fold is recomputed when one of its three parameters changes
+    with torch.no_grad():
+        net.encoder.fwd[2].weight.mul_(1.5)
+    y2, _ = run(True)
+    net.fold_encoder = False
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y2_layers = net(x.cuda())
+    net.fold_encoder = True
+    assert rel_l2(y2.float().cpu().numpy(), y2_layers.float().cpu().numpy()) < 2e-2
+    assert rel_l2(y2.float().cpu().numpy(), y_fold.float().cpu().numpy()) > 5e-2
+    # not applicable with repeated layers: block 0 then also receives a later block's output
+    for kw in (dict(repeat_layers=2),):
+        other = build(**{**case, **kw}).cuda().eval()
+        with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+            y = other(x.cuda())
+        assert other._fold_cache is None and torch.isfinite(y.float()).all()

@@ -535,6 +535,9 @@ def sfno_kernel_classes(dev, net, iters=10):
     # 1x1 convolutions of the pointwise tail: (name, module weight, bias, act, addend?, resolution, calls)
     hw_big, hw_small = net.inp_shape, (net.h, net.w)
     blk, last = net.blocks[1], net.blocks[-1]
+    # the last block's skip convolution and the decoder's first convolution run as one convolution over two tensors where the
+    # network merges them
+    merged = 1 if net._decoder_merge_ok() else 0
     convs = [("conv 73->384 +GELU 721x1440", net.encoder.fwd[0], "gelu", False, hw_big, 1),
              # the encoder's last convolution runs only where the network does not fold it into the first block's spectral weight
              ("conv 384->384 721x1440", net.encoder.fwd[2], None, False, hw_big, 0 if net._encoder_fold() is not None else 1),
@@ -543,8 +546,8 @@ def sfno_kernel_classes(dev, net, iters=10):
              ("conv 384->384 +addend 240x480", blk.outer_skip, None, True, hw_small, nl - 1),
              ("conv 384->768 +GELU 721x1440", last.mlp.fwd[0], "gelu", False, hw_big, 1),
              ("conv 768->384 721x1440", last.mlp.fwd[3], None, False, hw_big, 1),
-             ("conv 384->384 +addend 721x1440", last.outer_skip, None, True, hw_big, 1),
-             ("conv 384->384 +GELU 721x1440", net.decoder.fwd[0], "gelu", False, hw_big, 1),
+             ("conv 384->384 +addend 721x1440", last.outer_skip, None, True, hw_big, 1 - merged),
+             ("conv 384->384 +GELU 721x1440", net.decoder.fwd[0], "gelu", False, hw_big, 1 - merged),
              ("conv 384->73 +addend 721x1440", net.decoder.fwd[2], None, True, hw_big, 1),
              ("conv 73->73 721x1440", net.residual_transform, None, False, hw_big, 1)]
     for name, mod, act, add, (h, w_), calls in convs:
@@ -557,6 +560,16 @@ def sfno_kernel_classes(dev, net, iters=10):
         npx = h * w_
         mfma(name, calls, t, 2.0 * K * O * npx, 2 * npx * (K + O + (O if add else 0)))
         del xin, addend
+    if True:
+        h, w_ = hw_big
+        O, K = net.decoder.fwd[0].weight.shape[0], net.decoder.fwd[0].weight.shape[1]
+        x1 = torch.randn(1, K, h, w_, device=dev).to(torch.bfloat16)
+        x2 = torch.randn(1, K, h, w_, device=dev).to(torch.bfloat16)
+        wcat = torch.randn(O, 2 * K, device=dev) / (2 * K) ** 0.5
+        bias = torch.zeros(O, device=dev)
+        t = event_time_ms(lambda: pw.conv1x1_cat(x1, x2, wcat, bias, "gelu"), iters, stream)
+        mfma("conv (384+384)->384 +GELU 721x1440, two inputs", merged, t, 2.0 * 2 * K * O * h * w_, 2 * h * w_ * (2 * K + O))
+        del x1, x2
     # instance-norm statistics and the scale/shift/GELU pass
     for tag, (h, w_), calls in (("240x480", hw_small, nl - 1), ("721x1440", hw_big, 1)):
         xin = torch.randn(1, C, h, w_, device=dev).to(torch.bfloat16)

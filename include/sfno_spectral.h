@@ -290,6 +290,15 @@ int sfno_pointwise_conv(const void* x, const void* w, const float* bias, void* y
                         int64_t P, int act, const void* addend, const float* add_scale, const float* add_shift,
                         void* stream);
 
+/* The same convolution over the channel-wise concatenation of two tensors, without building it:
+ *   y[b][o][p] = act( sum_{k<K1} w[o][k] x1[b][k][p] + sum_{k<K2} w[o][K1+k] x2[b][k][p] + bias[o] )
+ * x1 bf16 [B][K1][P], x2 bf16 [B][K2][P], w packed from a float32 [O][K1+K2] matrix; more than 96 output channels
+ * (SFNO_EUNSUPPORTED otherwise).  No counterpart in the reference, which would run torch.cat and a Conv2d; used where two
+ * consecutive linear layers around a sum are merged into one (makani/models/networks/sfnonet.py:258-262 followed by
+ * makani/models/common/layers.py:95-116). */
+int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, int K2, const void* w, const float* bias, void* y,
+                            int batch, int O, int64_t P, int act, void* stream);
+
 /* Packs a 1x1 convolution weight (float32 [O][K], the nn.Conv2d parameter viewed as a matrix) into the bf16
  * MFMA operand stream sfno_pointwise_conv reads; `packed` holds sfno_pointwise_weight_elems(O, K) bf16 values. */
 int64_t sfno_pointwise_weight_elems(int O, int K);

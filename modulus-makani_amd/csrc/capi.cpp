@@ -575,6 +575,22 @@ extern "C" int sfno_pointwise_conv(const void* x, const void* w, const float* bi
     return pointwise_gemm_launch(a, (hipStream_t)stream);
 }
 
+extern "C" int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, int K2, const void* w, const float* bias, void* y, int batch,
+                                       int O, int64_t P, int act, void* stream) {
+    if (!x1 || !x2 || !w || !y || batch < 1 || K1 < 1 || K2 < 1 || O < 1 || P < 1) return SFNO_EINVAL;
+    if (act != SFNO_ACT_NONE && act != SFNO_ACT_GELU) return SFNO_EINVAL;
+    PointwiseArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.X = reinterpret_cast<const unsigned short*>(x1);
+    a.X2 = reinterpret_cast<const unsigned short*>(x2);
+    a.K1 = K1;
+    a.W = reinterpret_cast<const unsigned short*>(w);
+    a.bias = bias;
+    a.Y = reinterpret_cast<unsigned short*>(y);
+    a.K = K1 + K2; a.O = O; a.B = batch; a.act = act; a.P = P;
+    return pointwise_gemm_launch(a, (hipStream_t)stream);
+}
+
 extern "C" size_t sfno_instance_norm_workspace_bytes(int64_t rows, int64_t P) {
     if (rows < 1 || P < 1) return 0;
     return sizeof(float2) * (size_t)rows * row_stats_segments(rows, P);

@@ -283,7 +283,11 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
     const int nchunks = a.Kpad / DM_CK;
     const unsigned short* wsrc = a.W + (((int64_t)(ob * (DM_ROWS / 32) + 3 * (wave & 3)) * nc16 + (wave >> 2)) * 64 + lane) * 8;
     const int64_t wrb = (int64_t)nc16 * 512;                   // ushorts between row blocks
-    const unsigned short* __restrict__ X = a.X + (int64_t)b * a.K * a.P + min(pw0 + 8 * (lane & 31), a.P - 8);
+    // input channels k < K1 come from X, the others (if any) from X2: a convolution over the concatenation of two tensors
+    const int K1 = a.X2 ? a.K1 : a.K;
+    const int64_t xpx = min(pw0 + 8 * (lane & 31), a.P - 8);
+    const unsigned short* __restrict__ X = a.X + (int64_t)b * K1 * a.P + xpx;
+    const unsigned short* __restrict__ X2 = a.X2 ? a.X2 + (int64_t)b * (a.K - K1) * a.P + xpx : X;
     const int xrow0 = 4 * wave + (lane >> 5);                   // first of this lane's rows in the chunk: 2 (2 wave + i) + (lane >> 5)
 
     auto issue = [&](int c, int stage) {
@@ -294,7 +298,7 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int k = min(c * DM_CK + xrow0 + 2 * i, a.K - 1);      // rows past K meet zero weights
-            dma16(X + (int64_t)k * a.P, sb + DM_ABYTES + (2 * wave + i) * DM_XBLK);
+            dma16(k < K1 ? X + (int64_t)k * a.P : X2 + (int64_t)(k - K1) * a.P, sb + DM_ABYTES + (2 * wave + i) * DM_XBLK);
         }
     };
 
@@ -559,6 +563,7 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
     const bool tall = a.O > PW_ROWS;              // several wavefronts share a pixel strip
     const int wm = tall ? 4 : 1;
     const bool dma = tall;                        // direct-to-LDS kernel for O > 96
+    if (a.X2 && (!dma || a.K1 < 1 || a.K1 >= a.K)) return SFNO_EUNSUPPORTED;     // two input tensors: the tall kernel only
     const int wpx = dma ? DM_PX : 512;            // pixels per workgroup
     a.n_oblk = (a.O + PW_ROWS * wm - 1) / (PW_ROWS * wm);
     a.n_strips = (a.P + wpx - 1) / wpx;

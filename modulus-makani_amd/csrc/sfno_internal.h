@@ -73,7 +73,9 @@ int diagonal_wgrad_launch(const float2* x, const float2* g, float2* gw, int B, i
 
 // ---- pointwise tail (pointwise.hip): bf16 NCHW activations, 1x1 convolutions on bf16 MFMA ------------
 struct PointwiseArgs {
-    const unsigned short* X;       // bf16 [B][K][P]
+    const unsigned short* X;       // bf16 [B][K][P]; with X2: [B][K1][P], the first K1 input channels
+    const unsigned short* X2;      // null, or bf16 [B][K - K1][P]: the remaining input channels come from a second tensor
+    int K1;
     const unsigned short* W;       // packed by pointwise_pack_launch
     const float* bias;             // [O] or null
     unsigned short* Y;             // bf16 [B][O][P]

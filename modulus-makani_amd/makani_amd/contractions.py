@@ -29,7 +29,7 @@ class PackedWeights:
         """Re-pack if the parameter changed (in-place updates bump ``_version``).
 
         adjoint: this handle has shape (O, I, L) and is filled with the conjugate transpose of ``weight`` [I, O, L]."""
-        stamp = (weight.data_ptr(), weight._version)
+        stamp = (weight.data_ptr(), -1 if weight.is_inference() else weight._version)
         if stamp != self.stamp:
             w = weight.detach()
             if w.dtype != torch.complex64:

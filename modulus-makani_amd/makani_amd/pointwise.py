@@ -32,7 +32,8 @@ def packed_weight(weight):
     """MFMA operand stream of a 1x1 convolution weight ([O, K, 1, 1] or [O, K]); cached per parameter and
     rebuilt when the parameter changes."""
     key = id(weight)
-    stamp = (weight.data_ptr(), weight._version, weight.device)
+    # (tensors made under inference_mode carry no version counter: they are packed once per tensor object)
+    stamp = (weight.data_ptr(), -1 if weight.is_inference() else weight._version, weight.device)
     hit = _wcache.get(key)
     if hit is not None and hit[0]() is weight and hit[1] == stamp:
         return hit[2]
@@ -84,6 +85,26 @@ def conv1x1(x, weight, bias=None, act=None, addend=None, add_scale=None, add_shi
                                 _ptr(add_shift), _stream(x.device)),
         "sfno_pointwise_conv",
     )
+    return y
+
+
+def conv1x1_cat(x1, x2, weight, bias=None, act=None):
+    """act(conv1x1(cat([x1, x2], dim=1), weight) + bias) without building the concatenation  ->  bf16 [B, O, H, W];
+    weight [O, K1 + K2] (or [O, K1 + K2, 1, 1]), more than 96 output channels."""
+    if not (supported(x1) and supported(x2)) or x1.shape[0] != x2.shape[0] or x1.shape[2:] != x2.shape[2:]:
+        raise RuntimeError("conv1x1_cat takes two contiguous bfloat16 NCHW HIP tensors of one batch and grid size, H*W a multiple of 8")
+    x1, x2 = x1.contiguous(), x2.contiguous()
+    B, K1, H, W = x1.shape
+    K2 = x2.shape[1]
+    O = weight.shape[0]
+    if weight.reshape(O, -1).shape[1] != K1 + K2:
+        raise RuntimeError(f"conv1x1_cat: inputs have {K1} + {K2} channels, weight expects {weight.reshape(O, -1).shape[1]}")
+    pw = packed_weight(weight)
+    y = torch.empty((B, O, H, W), dtype=torch.bfloat16, device=x1.device)
+    if bias is not None:
+        bias = bias.detach().float().contiguous()
+    check(lib.sfno_pointwise_conv_cat(_ptr(x1), K1, _ptr(x2), K2, _ptr(pw), _ptr(bias), _ptr(y), B, O, H * W, ACT[act], _stream(x1.device)),
+          "sfno_pointwise_conv_cat")
     return y
 
 

@@ -190,7 +190,7 @@ class FourierNeuralOperatorBlock(nn.Module):
             return False
         return hasattr(self, "outer_skip") and _is_conv1x1(self.outer_skip) and self.outer_skip.bias is None
 
-    def _forward_fused(self, x, residual, lat_stats=None, skip_weight=None):
+    def _forward_fused(self, x, residual, lat_stats=None, skip_weight=None, defer_skip=False):
         """norm0 -> GELU -> MLP -> norm1 -> + outer_skip(residual) in five kernels: row statistics (or, for norm0, the
         per-latitude moments the inverse transform delivered with x), scale/shift + GELU, two 1x1 convolutions with bias
         (+ GELU) epilogues, row statistics, and the skip convolution whose epilogue adds the normalised MLP output."""
@@ -205,11 +205,14 @@ class FourierNeuralOperatorBlock(nn.Module):
         x = pw.scale_shift_act(x, sc, sh, "gelu")
         x = _run_chain(_fused_chain(self.mlp.fwd), x)
         sc, sh = _norm_coeffs(self.norm1, x)
+        if defer_skip:
+            # the caller merges "norm1(x) + outer_skip(residual)" into the linear layer that follows (the network's _decoder_merge)
+            return x, residual, sc, sh
         # skip_weight: the skip convolution composed with a linear map the caller pulled out of `residual` (see the network's
         # _encoder_fold)
         return pw.conv1x1(residual, self.outer_skip.weight if skip_weight is None else skip_weight, None, None, x, sc, sh)
 
-    def forward(self, x):
+    def forward(self, x, defer_skip=False):
         # on the fused inference path the inverse transform hands over the moments norm0 needs together with its output
         want_stats = getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and self._fusable()
         if want_stats:
@@ -218,7 +221,8 @@ class FourierNeuralOperatorBlock(nn.Module):
             (x, residual), lat_stats = self.filter(x), None
         if getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 \
                 and residual.shape[2:] == x.shape[2:] and self._fusable():
-            return self._forward_fused(x.contiguous(), residual.contiguous(), lat_stats)
+            return self._forward_fused(x.contiguous(), residual.contiguous(), lat_stats, defer_skip=defer_skip)
+        # (defer_skip is honoured on the fused path only; here the block's output comes back whole)
         x = self.norm0(x)
         if hasattr(self, "inner_skip"):
             x = x + self.inner_skip(residual)
@@ -242,12 +246,16 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                  encoder_layers=1, pos_embed="none", pos_drop_rate=0.0, path_drop_rate=0.0, mlp_drop_rate=0.0,
                  normalization_layer="instance_norm", max_modes=None, hard_thresholding_fraction=1.0, big_skip=True, rank=1.0,
                  factorization=None, separable=False, complex_activation="real", spectral_layers=3, bias=False, checkpointing=0,
-                 spectral_compute="fp32", fused_pointwise=True, fold_encoder=True, **kwargs):
+                 spectral_compute="fp32", fused_pointwise=True, fold_encoder=True, merge_decoder=True, **kwargs):
         super().__init__()
         # fold_encoder (not a Makani option): on the fused inference path the encoder's last (linear) convolution is applied in
         # spectral space, inside the first block's weights, instead of at full resolution; see _encoder_fold
         self.fold_encoder = fold_encoder
         self._fold_cache = None
+        # merge_decoder (not a Makani option): on the same path the last block's skip convolution and norm1 are merged into the
+        # decoder's first convolution; see _decoder_merge_ok
+        self.merge_decoder = merge_decoder
+        self._merge_cache = None
         # fused_pointwise (not a Makani option): under torch.no_grad() / inference_mode() with bf16 autocast the 1x1 convolutions,
         # instance norms and GELUs run on the fused HIP kernels (weights rounded to bf16 once, fp32 accumulation, one rounding per
         # layer, norm0 statistics from the unrounded field).  A forward that records gradients always runs the PyTorch modules, so
@@ -386,6 +394,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         """Forgets the folded weights (they follow in-place updates of their three parameters through the version counters;
         call this after writing one of them through ``.data``)."""
         self._fold_cache = None
+        self._merge_cache = None
 
     def _block0_folded(self, h, wf, wsk):
         blk = self.blocks[0]
@@ -396,6 +405,54 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         spec = dhconv_spectral(spec, wf, B, conv.modes_lon, triangular=conv._triangular, compute=conv.compute)
         x, stats = conv.inverse_transform.synthesis_with_lat_stats(spec, (B, conv.out_channels), dtype=torch.bfloat16)
         return blk._forward_fused(x.contiguous(), residual.contiguous(), stats, skip_weight=wsk)
+
+    # The last block ends in  x = scale * m + shift + W_skip r  (norm1 of the MLP output m as a per-(sample, channel) affine, plus
+    # the skip convolution of the residual r) and nothing but the decoder's first convolution W_d, b_d reads x.  Both steps are
+    # linear, so they are one convolution over the two tensors m and r, with the weight [W_d diag(scale) | W_d W_skip] and the
+    # bias W_d shift + b_d of each sample: the sum is never written and the skip convolution's 384 x 384 products per pixel at
+    # full resolution are not computed.  W_d and W_skip enter with their bf16-rounded values, as autocast would use them.
+    def _decoder_merge_ok(self):
+        if not getattr(self, "merge_decoder", True) or self.repeat_layers != 1 or len(self.blocks) < 2:
+            return False
+        dec = _fused_chain(self.decoder.fwd)
+        blk = self.blocks[-1]
+        if dec is None or not (isinstance(blk, FourierNeuralOperatorBlock) and blk._fusable() and getattr(blk, "fused_pointwise", True)):
+            return False
+        wd = dec[0][0].weight
+        return wd.shape[0] > 96 and wd.shape[1] == blk.outer_skip.weight.shape[0]
+
+    def _decoder_merged(self, x):
+        """Last block and the decoder's first step for the output x of the block before it; returns the result and the decoder
+        steps still to run."""
+        blk, dec = self.blocks[-1], _fused_chain(self.decoder.fwd)
+        conv_d = dec[0][0]
+        out = blk(x, defer_skip=True)
+        if not isinstance(out, tuple):           # the block could not take its fused path after all: layer by layer from here
+            return out, dec
+        m, r, sc, sh = out
+        B, C = m.shape[:2]
+        with torch.inference_mode(False), torch.no_grad():
+            cached = getattr(self, "_merge_cache", None)
+            stamp = tuple((t.data_ptr(), t._version) for t in (conv_d.weight, blk.outer_skip.weight))
+            if cached is None or cached[0] != stamp:
+                wd = conv_d.weight.detach().reshape(conv_d.weight.shape[0], -1).to(torch.bfloat16).float()
+                ws = blk.outer_skip.weight.detach().reshape(C, -1).to(torch.bfloat16).float()
+                cached = (stamp, wd, (wd @ ws).contiguous())
+                self._merge_cache = cached
+            wd, wds = cached[1], cached[2]
+            if sc is None:
+                sc = torch.ones((B, C), dtype=torch.float32, device=m.device)
+                sh = torch.zeros_like(sc)
+            sc, sh = sc.clone(), sh.clone()          # ordinary tensors for the arithmetic below
+            outs = []
+            for b in range(B):
+                wcat = torch.cat([wd * sc[b][None, :], wds], dim=1).contiguous()
+                bias = wd @ sh[b]
+                if conv_d.bias is not None:
+                    bias = bias + conv_d.bias.detach().float()
+                outs.append((wcat, bias))
+        ys = [pw.conv1x1_cat(m[b:b + 1], r[b:b + 1], wcat, bias, dec[0][1]) for b, (wcat, bias) in enumerate(outs)]
+        return (ys[0] if B == 1 else torch.cat(ys, dim=0)), dec[1:]
 
     def _forward_fused(self, x):
         """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""
@@ -408,13 +465,23 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                 residual = xb
             residual = pw.conv1x1(residual, self.residual_transform.weight)
         fold = self._encoder_fold()
+        merge = self._decoder_merge_ok()
         if fold is not None:
             x = self._block0_folded(_run_chain(fold[0], xb), fold[1], fold[2])
-            for blk in self.blocks[1:]:
-                x = blk(x)
+            rest = self.blocks[1:]
+        elif merge:
+            x = _run_chain(enc, xb)
+            rest = self.blocks
         else:
             x = _run_chain(enc, xb)
             x = self._forward_features(x)
+            rest = []
+        for blk in (rest[:-1] if merge else rest):
+            x = blk(x)
+        if merge:
+            x, dec = self._decoder_merged(x.to(torch.bfloat16).contiguous())
+            if not dec:
+                return x + residual if self.big_skip else x
         return _run_chain(dec, x.to(torch.bfloat16).contiguous(), residual if self.big_skip else None)
 
     def _fusable(self, x):

@@ -249,3 +249,40 @@ def test_encoder_fold_matches_layer_by_layer(lib_built):
         with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
             y = other(x.cuda())
         assert other._fold_cache is None and torch.isfinite(y.float()).all()
+
+
+def test_decoder_merge_matches_layer_by_layer(lib_built):
+    """merge_decoder: the last block's "norm1(mlp) + outer_skip(residual)" and the decoder's first convolution are one convolution
+    over the two tensors (both steps are linear), with per-sample weights [W_d diag(scale) | W_d W_skip] and bias W_d shift + b_d.
+    Same network, merged against layer by layer, through the float64 oracle model; batch 2, so that the per-sample weights differ."""
+    case = dict(inp_shape=(92, 180), out_shape=(92, 180), inp_chans=5, out_chans=5, scale_factor=3, embed_dim=128, num_layers=3)
+    print(f"case sfno decoder merge {case}", flush=True)
+    net = build(**case).cuda().eval()
+    g = torch.Generator().manual_seed(12)
+    with torch.no_grad():
+        for n, p in net.named_parameters():
+            if "norm" in n or n.endswith(".bias"):
+                p.add_(0.3 * torch.randn(p.shape, generator=g).to(p.device))
+    x = torch.randn(2, 5, 92, 180, generator=torch.Generator().manual_seed(8))
+    x[1] *= 3.0
+
+    def run(merge):
+        net.merge_decoder = merge
+        net._merge_cache = None
+        with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+            y = net(x.cuda())
+        return y, net._merge_cache is not None
+
+    (y_m, taken), (y_l, taken_off) = run(True), run(False)
+    assert taken and not taken_off
+    ref64 = SfnoOracle((92, 180), (92, 180), 3, 3).forward(net.state_dict(), x).numpy()
+    e_m = rel_l2(y_m.float().cpu().double().numpy(), ref64)
+    e_l = rel_l2(y_l.float().cpu().double().numpy(), ref64)
+    d = rel_l2(y_m.float().cpu().numpy(), y_l.float().cpu().numpy())
+    print(f"merged {e_m:.3e}  layer by layer {e_l:.3e}  between them {d:.3e}", flush=True)
+    assert e_m < 2e-2 and e_m < 1.1 * e_l and d < e_m + e_l
+    # narrow decoders (at most 96 channels) keep the layer-by-layer evaluation
+    small = build(**{**case, "embed_dim": 48}).cuda().eval()
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = small(x.cuda())
+    assert small._merge_cache is None and torch.isfinite(y.float()).all()

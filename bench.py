@@ -538,6 +538,8 @@ def sfno_kernel_classes(dev, net, iters=10):
     # the last block's skip convolution and the decoder's first convolution run as one convolution over two tensors where the
     # network merges them
     merged = 1 if net._decoder_merge_ok() else 0
+    # likewise the decoder's last convolution and the convolution of the big skip
+    tail = 1 if net._tail_cat_ok() else 0
     convs = [("conv 73->384 +GELU 721x1440", net.encoder.fwd[0], "gelu", False, hw_big, 1),
              # the encoder's last convolution runs only where the network does not fold it into the first block's spectral weight
              ("conv 384->384 721x1440", net.encoder.fwd[2], None, False, hw_big, 0 if net._encoder_fold() is not None else 1),
@@ -548,8 +550,8 @@ def sfno_kernel_classes(dev, net, iters=10):
              ("conv 768->384 721x1440", last.mlp.fwd[3], None, False, hw_big, 1),
              ("conv 384->384 +addend 721x1440", last.outer_skip, None, True, hw_big, 1 - merged),
              ("conv 384->384 +GELU 721x1440", net.decoder.fwd[0], "gelu", False, hw_big, 1 - merged),
-             ("conv 384->73 +addend 721x1440", net.decoder.fwd[2], None, True, hw_big, 1),
-             ("conv 73->73 721x1440", net.residual_transform, None, False, hw_big, 1)]
+             ("conv 384->73 +addend 721x1440", net.decoder.fwd[2], None, True, hw_big, 1 - tail),
+             ("conv 73->73 721x1440", net.residual_transform, None, False, hw_big, 1 - tail)]
     for name, mod, act, add, (h, w_), calls in convs:
         O, K = mod.weight.shape[0], mod.weight.shape[1]
         xin = torch.randn(1, K, h, w_, device=dev).to(torch.bfloat16)
@@ -569,6 +571,13 @@ def sfno_kernel_classes(dev, net, iters=10):
         bias = torch.zeros(O, device=dev)
         t = event_time_ms(lambda: pw.conv1x1_cat(x1, x2, wcat, bias, "gelu"), iters, stream)
         mfma("conv (384+384)->384 +GELU 721x1440, two inputs", merged, t, 2.0 * 2 * K * O * h * w_, 2 * h * w_ * (2 * K + O))
+        del x1, x2
+        O, K, K2 = net.decoder.fwd[2].weight.shape[0], net.decoder.fwd[2].weight.shape[1], net.residual_transform.weight.shape[1]
+        x1 = torch.randn(1, K, h, w_, device=dev).to(torch.bfloat16)
+        x2 = torch.randn(1, K2, h, w_, device=dev).to(torch.bfloat16)
+        wcat = torch.randn(O, K + K2, device=dev) / (K + K2) ** 0.5
+        t = event_time_ms(lambda: pw.conv1x1_cat(x1, x2, wcat, None, None), iters, stream)
+        mfma("conv (384+73)->73 721x1440, two inputs", tail, t, 2.0 * (K + K2) * O * h * w_, 2 * h * w_ * (K + K2 + O))
         del x1, x2
     # instance-norm statistics and the scale/shift/GELU pass
     for tag, (h, w_), calls in (("240x480", hw_small, nl - 1), ("721x1440", hw_big, 1)):

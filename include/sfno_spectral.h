@@ -292,10 +292,10 @@ int sfno_pointwise_conv(const void* x, const void* w, const float* bias, void* y
 
 /* The same convolution over the channel-wise concatenation of two tensors, without building it:
  *   y[b][o][p] = act( sum_{k<K1} w[o][k] x1[b][k][p] + sum_{k<K2} w[o][K1+k] x2[b][k][p] + bias[o] )
- * x1 bf16 [B][K1][P], x2 bf16 [B][K2][P], w packed from a float32 [O][K1+K2] matrix; more than 96 output channels
- * (SFNO_EUNSUPPORTED otherwise).  No counterpart in the reference, which would run torch.cat and a Conv2d; used where two
+ * x1 bf16 [B][K1][P], x2 bf16 [B][K2][P], w packed from a float32 [O][K1+K2] matrix.  No counterpart in the reference, which would run torch.cat and a Conv2d; used where two
  * consecutive linear layers around a sum are merged into one (makani/models/networks/sfnonet.py:258-262 followed by
- * makani/models/common/layers.py:95-116). */
+ * makani/models/common/layers.py:95-116) and where two convolutions feed one sum (decoder output + residual_transform
+ * of the input, sfnonet.py:636-638). */
 int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, int K2, const void* w, const float* bias, void* y,
                             int batch, int O, int64_t P, int act, void* stream);
 

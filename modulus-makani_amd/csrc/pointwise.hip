@@ -84,7 +84,10 @@ __global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseA
     const int o0 = ob * (PW_ROWS * WM) + (wave / WN) * PW_ROWS;
     const int pxw = (wave % WN) * PW_PX;                                  // wavefront's pixel offset inside the stage
 
-    const unsigned short* __restrict__ X = a.X + (int64_t)b * a.K * a.P;
+    // input channels k < K1 come from X, the others (if any) from X2: a convolution over the concatenation of two tensors
+    const int K1 = a.X2 ? a.K1 : a.K;
+    const unsigned short* __restrict__ X = a.X + (int64_t)b * K1 * a.P;
+    const unsigned short* __restrict__ X2 = a.X2 ? a.X2 + (int64_t)b * (a.K - K1) * a.P : X;
     // this thread's 16-byte pieces (8 pixels of one k row) of an activation chunk of CK rows x WPX pixels
     int xr[XW], loff[XW];
     int64_t xoff[XW];
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseA
 #pragma unroll
         for (int u = 0; u < XW; ++u) {
             const int k = min(cc * CK + xr[u], a.K - 1);                  // rows past K meet zero weights
-            dst[u] = *reinterpret_cast<const u32x4*>(X + (int64_t)k * a.P + xoff[u]);
+            dst[u] = *reinterpret_cast<const u32x4*>((k < K1 ? X + (int64_t)k * a.P : X2 + (int64_t)(k - K1) * a.P) + xoff[u]);
         }
     };
     auto store_x = [&](int stage, const u32x4 (&src)[XW]) {
@@ -563,7 +566,7 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
     const bool tall = a.O > PW_ROWS;              // several wavefronts share a pixel strip
     const int wm = tall ? 4 : 1;
     const bool dma = tall;                        // direct-to-LDS kernel for O > 96
-    if (a.X2 && (!dma || a.K1 < 1 || a.K1 >= a.K)) return SFNO_EUNSUPPORTED;     // two input tensors: the tall kernel only
+    if (a.X2 && (a.K1 < 1 || a.K1 >= a.K)) return SFNO_EINVAL;
     const int wpx = dma ? DM_PX : 512;            // pixels per workgroup
     a.n_oblk = (a.O + PW_ROWS * wm - 1) / (PW_ROWS * wm);
     a.n_strips = (a.P + wpx - 1) / wpx;

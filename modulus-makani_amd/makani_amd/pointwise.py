@@ -90,7 +90,7 @@ def conv1x1(x, weight, bias=None, act=None, addend=None, add_scale=None, add_shi
 
 def conv1x1_cat(x1, x2, weight, bias=None, act=None):
     """act(conv1x1(cat([x1, x2], dim=1), weight) + bias) without building the concatenation  ->  bf16 [B, O, H, W];
-    weight [O, K1 + K2] (or [O, K1 + K2, 1, 1]), more than 96 output channels."""
+    weight [O, K1 + K2] (or [O, K1 + K2, 1, 1])."""
     if not (supported(x1) and supported(x2)) or x1.shape[0] != x2.shape[0] or x1.shape[2:] != x2.shape[2:]:
         raise RuntimeError("conv1x1_cat takes two contiguous bfloat16 NCHW HIP tensors of one batch and grid size, H*W a multiple of 8")
     x1, x2 = x1.contiguous(), x2.contiguous()

@@ -256,6 +256,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         # decoder's first convolution; see _decoder_merge_ok
         self.merge_decoder = merge_decoder
         self._merge_cache = None
+        self._tail_cache = None
         # fused_pointwise (not a Makani option): under torch.no_grad() / inference_mode() with bf16 autocast the 1x1 convolutions,
         # instance norms and GELUs run on the fused HIP kernels (weights rounded to bf16 once, fp32 accumulation, one rounding per
         # layer, norm0 statistics from the unrounded field).  A forward that records gradients always runs the PyTorch modules, so
@@ -395,6 +396,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         call this after writing one of them through ``.data``)."""
         self._fold_cache = None
         self._merge_cache = None
+        self._tail_cache = None
 
     def _block0_folded(self, h, wf, wsk):
         blk = self.blocks[0]
@@ -420,6 +422,22 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
             return False
         wd = dec[0][0].weight
         return wd.shape[0] > 96 and wd.shape[1] == blk.outer_skip.weight.shape[0]
+
+    def _tail_cat_ok(self):
+        dec = _fused_chain(self.decoder.fwd)
+        return bool(self.big_skip and getattr(self, "merge_decoder", True) and dec and dec[-1][1] is None)
+
+    def _tail_weight(self, conv):
+        """[W_last | W_res] of the decoder's last convolution and residual_transform, cached until one of them changes."""
+        wl, wr = conv.weight, self.residual_transform.weight
+        stamp = tuple((t.data_ptr(), t._version) for t in (wl, wr))
+        cached = getattr(self, "_tail_cache", None)
+        if cached is None or cached[0] != stamp:
+            with torch.inference_mode(False), torch.no_grad():
+                w = torch.cat([wl.detach().reshape(wl.shape[0], -1).float(), wr.detach().reshape(wr.shape[0], -1).float()], dim=1).contiguous()
+            cached = (stamp, w)
+            self._tail_cache = cached
+        return cached[1]
 
     def _decoder_merged(self, x):
         """Last block and the decoder's first step for the output x of the block before it; returns the result and the decoder
@@ -458,12 +476,17 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""
         enc, dec = _fused_chain(self.encoder.fwd), _fused_chain(self.decoder.fwd)
         xb = x.to(torch.bfloat16).contiguous()
+        cat_tail = False
         if self.big_skip:
             if self.out_shape != self.inp_shape:
                 residual = self.itrans_up(self.trans_down(x.to(torch.float32)).contiguous()).to(torch.bfloat16).contiguous()
             else:
                 residual = xb
-            residual = pw.conv1x1(residual, self.residual_transform.weight)
+            # the decoder's last convolution and residual_transform feed one sum (sfnonet.py:636-638): one convolution over
+            # the two tensors with the weight [W_last | W_res]; where that does not apply the residual is convolved here
+            cat_tail = self._tail_cat_ok()
+            if not cat_tail:
+                residual = pw.conv1x1(residual, self.residual_transform.weight)
         fold = self._encoder_fold()
         merge = self._decoder_merge_ok()
         if fold is not None:
@@ -480,9 +503,16 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
             x = blk(x)
         if merge:
             x, dec = self._decoder_merged(x.to(torch.bfloat16).contiguous())
-            if not dec:
-                return x + residual if self.big_skip else x
-        return _run_chain(dec, x.to(torch.bfloat16).contiguous(), residual if self.big_skip else None)
+        x = x.to(torch.bfloat16).contiguous()
+        if self.big_skip and cat_tail:
+            if not dec:                           # the merged convolution was the decoder's last step: the residual is still to be added
+                return x + pw.conv1x1(residual, self.residual_transform.weight)
+            x = _run_chain(dec[:-1], x)
+            conv = dec[-1][0]
+            return pw.conv1x1_cat(x, residual, self._tail_weight(conv), conv.bias, None)
+        if not dec:
+            return x + residual if self.big_skip else x
+        return _run_chain(dec, x, residual if self.big_skip else None)
 
     def _fusable(self, x):
         if not (getattr(self, "fused_pointwise", True) and fused_pointwise_active(x)) or hasattr(self, "pos_embed"):

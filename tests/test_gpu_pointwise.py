@@ -219,11 +219,12 @@ def test_latitude_moments_against_statistics_of_the_rounded_field(lib_built, nla
 
 def test_conv1x1_over_two_tensors(lib_built):
     """sfno_pointwise_conv_cat: the convolution over the channel-wise concatenation of two tensors equals the convolution of the
-    concatenated tensor (same kernel, same order of the sum: bit for bit), with bias and GELU, K1 and K2 not multiples of the chunk."""
+    concatenated tensor (same kernel, same order of the sum: bit for bit), with bias and GELU, K1 and K2 not multiples of the chunk,
+    on both kernels (more and at most 96 output channels)."""
     from makani_amd import pointwise as pw
 
     g = torch.Generator().manual_seed(21)
-    for (B, K1, K2, O, H, W) in ((1, 384, 384, 384, 24, 40), (2, 50, 77, 128, 16, 24), (1, 32, 416, 200, 8, 64)):
+    for (B, K1, K2, O, H, W) in ((1, 384, 384, 384, 24, 40), (2, 50, 77, 128, 16, 24), (1, 32, 416, 200, 8, 64), (2, 384, 73, 73, 16, 40), (1, 5, 3, 7, 8, 8)):
         x1 = torch.randn(B, K1, H, W, generator=g).bfloat16().cuda()
         x2 = torch.randn(B, K2, H, W, generator=g).bfloat16().cuda()
         w = (torch.randn(O, K1 + K2, generator=g) / (K1 + K2) ** 0.5).cuda()
@@ -233,4 +234,4 @@ def test_conv1x1_over_two_tensors(lib_built):
             want = pw.conv1x1(torch.cat([x1, x2], dim=1).contiguous(), w, bias, act)
             assert torch.equal(got, want), (B, K1, K2, O, act)
     with pytest.raises(RuntimeError):
-        pw.conv1x1_cat(x1, x2, torch.randn(64, K1 + K2).cuda())          # at most 96 output channels: not provided
+        pw.conv1x1_cat(x1, x2, torch.randn(64, K1 + K2 + 1).cuda())      # weight of another width

@@ -88,9 +88,9 @@ def conv1x1(x, weight, bias=None, act=None, addend=None, add_scale=None, add_shi
     return y
 
 
-def conv1x1_cat(x1, x2, weight, bias=None, act=None):
+def conv1x1_cat(x1, x2, weight, bias=None, act=None, out=None):
     """act(conv1x1(cat([x1, x2], dim=1), weight) + bias) without building the concatenation  ->  bf16 [B, O, H, W];
-    weight [O, K1 + K2] (or [O, K1 + K2, 1, 1])."""
+    weight [O, K1 + K2] (or [O, K1 + K2, 1, 1]); out: a contiguous bf16 tensor of the result's shape to write into."""
     if not (supported(x1) and supported(x2)) or x1.shape[0] != x2.shape[0] or x1.shape[2:] != x2.shape[2:]:
         raise RuntimeError("conv1x1_cat takes two contiguous bfloat16 NCHW HIP tensors of one batch and grid size, H*W a multiple of 8")
     x1, x2 = x1.contiguous(), x2.contiguous()
@@ -100,7 +100,12 @@ def conv1x1_cat(x1, x2, weight, bias=None, act=None):
     if weight.reshape(O, -1).shape[1] != K1 + K2:
         raise RuntimeError(f"conv1x1_cat: inputs have {K1} + {K2} channels, weight expects {weight.reshape(O, -1).shape[1]}")
     pw = packed_weight(weight)
-    y = torch.empty((B, O, H, W), dtype=torch.bfloat16, device=x1.device)
+    if out is None:
+        y = torch.empty((B, O, H, W), dtype=torch.bfloat16, device=x1.device)
+    else:
+        if tuple(out.shape) != (B, O, H, W) or out.dtype != torch.bfloat16 or not out.is_contiguous() or out.device != x1.device:
+            raise RuntimeError("conv1x1_cat: out must be a contiguous bfloat16 tensor of the result's shape")
+        y = out
     if bias is not None:
         bias = bias.detach().float().contiguous()
     check(lib.sfno_pointwise_conv_cat(_ptr(x1), K1, _ptr(x2), K2, _ptr(pw), _ptr(bias), _ptr(y), B, O, H * W, ACT[act], _stream(x1.device)),

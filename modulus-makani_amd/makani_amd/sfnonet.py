@@ -469,8 +469,10 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                 if conv_d.bias is not None:
                     bias = bias + conv_d.bias.detach().float()
                 outs.append((wcat, bias))
-        ys = [pw.conv1x1_cat(m[b:b + 1], r[b:b + 1], wcat, bias, dec[0][1]) for b, (wcat, bias) in enumerate(outs)]
-        return (ys[0] if B == 1 else torch.cat(ys, dim=0)), dec[1:]
+        y = torch.empty((B, wd.shape[0], m.shape[2], m.shape[3]), dtype=torch.bfloat16, device=m.device)
+        for b, (wcat, bias) in enumerate(outs):
+            pw.conv1x1_cat(m[b:b + 1], r[b:b + 1], wcat, bias, dec[0][1], out=y[b:b + 1])
+        return y, dec[1:]
 
     def _forward_fused(self, x):
         """Encoder, blocks and decoder with every 1x1 convolution on the fused bf16 kernels (inference under bf16 autocast)."""

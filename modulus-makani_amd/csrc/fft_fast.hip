@@ -839,7 +839,7 @@ struct FastEntry {
     int n, r0, r1, r2;
 };
 // lengths with a specialised kernel; the last radix acts on contiguous groups, an odd one keeps LDS banks apart
-const FastEntry kFast[] = {{1536, 16, 12, 8}, {1440, 16, 10, 9}, {1024, 16, 8, 8}, {720, 16, 5, 9}, {512, 8, 8, 8}, {480, 10, 16, 3}, {360, 8, 5, 9},
+const FastEntry kFast[] = {{1536, 16, 12, 8}, {1440, 16, 10, 9}, {1024, 16, 8, 8}, {720, 16, 5, 9}, {512, 8, 8, 8}, {480, 4, 8, 15}, {360, 8, 5, 9},
                            {256, 16, 16, 1}, {240, 16, 5, 3}, {180, 4, 5, 9}, {128, 8, 16, 1}, {64, 8, 8, 1}};
 
 const FastEntry* find_fast(int n) {
@@ -1006,7 +1006,7 @@ int latfft_fast_launch(bool inverse, const FftPlan& p, const float* in, float* o
         case 1024: return go_lat<1024, 16, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 720: return go_lat<720, 16, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 512: return go_lat<512, 8, 8, 8>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
-        case 480: return go_lat<480, 10, 16, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
+        case 480: return go_lat<480, 4, 8, 15>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 360: return go_lat<360, 8, 5, 9>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 256: return go_lat<256, 16, 16, 1>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
         case 240: return go_lat<240, 16, 5, 3>(inverse, p, in, out, mmax, lmax, ld, mscale, s);
@@ -1037,7 +1037,7 @@ int fft_fast_launch(bool inverse, const FftPlan& p, const void* in, void* out, i
         FF_CASE(1024, 16, 8, 8)
         FF_CASE(720, 16, 5, 9)
         FF_CASE(512, 8, 8, 8)
-        FF_CASE(480, 10, 16, 3)
+        FF_CASE(480, 4, 8, 15)
         FF_CASE(360, 8, 5, 9)
         FF_CASE(256, 16, 16, 1)
         FF_CASE(240, 16, 5, 3)

@@ -17,6 +17,7 @@
 // stage, both prefetched in registers.  All others (pw_gemm_dma_kernel, further down): 384 rows x 256 pixels per
 // workgroup with both operand streams loaded straight into LDS.
 #include "sfno_internal.h"
+#include <type_traits>
 
 namespace sfno {
 namespace {
@@ -34,6 +35,12 @@ constexpr int PW_KALIGN = 128;    // K is padded to whole unrolled loop bodies (
 
 __device__ __forceinline__ float bf16_to_f(unsigned short h) { return __uint_as_float((unsigned int)h << 16); }
 __device__ __forceinline__ unsigned short f_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
+
+// p[i] for a wavefront-uniform i, of an array the kernel never writes: read through the scalar unit, whose loads do not
+// count against the vector memory counter
+__device__ __forceinline__ float uniform_load(const float* p, int64_t i) {
+    return reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(p))[i];
+}
 
 // exact (erf) GELU for bf16 outputs.  gelu(x) = max(x, 0) - |x| erfc(|x| / sqrt 2) / 2 for both signs (no cancellation in
 // the negative tail), and erfc is evaluated as 2^Q(|x|): log2 erfc(t / sqrt 2) is smooth, a degree-7 polynomial in t follows it
@@ -247,62 +254,112 @@ __global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseA
 // For O > 96 the kernel above is bound by the weight fragments every wavefront pulls through L1 for only 6 MFMAs
 // each.  This variant gives a wavefront 96 rows x 128 pixels (3 x 4 tiles, 192 accumulator registers), eight
 // wavefronts per workgroup (384 rows x 256 pixels, half the weight traffic per pixel), and moves both operand
-// streams with global_load_lds_dwordx4: lane i's 16 bytes land at LDS base + 16 i, no staging registers, so three
-// stages of 32 k rows (40 KiB each) give a two-chunk prefetch distance within the 256 registers two wavefronts
-// per SIMD leave.  The loads are issued from inline assembly: the compiler would otherwise order every LDS read
-// behind all outstanding direct-to-LDS loads; the waits are written out by hand (5 loads per wavefront and chunk).
+// streams with global_load_lds_dwordx4: lane i's 16 bytes land at LDS base + 16 i, no staging registers.
+//
+// One persistent workgroup per CU walks its tiles as one unbroken stream of 32-row K chunks, so the operands of the
+// next tile are already in LDS when the stores of the current one leave.  A read only reaches the HBM rate with
+// some 50 KB in flight per CU, and the memory counter of a wavefront retires in order, so a wavefront that waits for
+// a weight block (an L2 hit) would also wait for every activation block it asked for earlier.  The two streams
+// therefore belong to different wavefronts: wavefronts 0-3 fetch the weights two chunks ahead (three stages of
+// 24 KiB), wavefronts 4-7 the activations four chunks ahead (five stages of 16 KiB: 64 KiB in flight).  The loads are
+// issued from inline assembly (the compiler would order every LDS read behind all outstanding direct-to-LDS loads)
+// and the waits are written out by hand.  Other memory operations of a wavefront (the epilogue's stores and addend
+// loads) are older than the loads a wait is meant for or younger than all of them; either way the wait covers
+// at least the loads it is meant for.
 constexpr int DM_MT = 3, DM_NT = 4;
 constexpr int DM_ROWS = 4 * 32 * DM_MT;          // 384 rows per workgroup
 constexpr int DM_PX = 2 * 32 * DM_NT;            // 256 pixels per workgroup
 constexpr int DM_CK = 32;                        // k rows per chunk
-constexpr int DM_ABYTES = 2 * (DM_ROWS / 32) * 1024;   // 24 fragment blocks of 1 KiB
+constexpr int DM_ABYTES = 2 * (DM_ROWS / 32) * 1024;   // weight stage: 24 fragment blocks of 1 KiB
 constexpr int DM_XBLK = 1024 + 16;               // two pixel rows of the chunk (2 x 512 bytes) + padding
-constexpr int DM_STAGE = DM_ABYTES + (DM_CK / 2) * DM_XBLK;
-constexpr int DM_NSTAGE = 3;
+constexpr int DM_XBYTES = (DM_CK / 2) * DM_XBLK; // activation stage
+constexpr int DM_WSTAGES = 3, DM_XSTAGES = 5;    // prefetch distance + 1
+constexpr int DM_XBASE = DM_WSTAGES * DM_ABYTES;
+constexpr int DM_LDS = DM_XBASE + DM_XSTAGES * DM_XBYTES;
+static_assert(DM_LDS <= 160 * 1024, "one workgroup per CU");
 
 __device__ __forceinline__ void dma16(const void* g, unsigned lds_byte_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_addr) : "memory");
 }
 
+// GELU: exact GELU on the output; ADD: "+ scale * addend + shift"
+template <bool GELU, bool ADD>
 __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
-    __shared__ __align__(16) unsigned char lds[DM_NSTAGE * DM_STAGE];
-    const int xcd = blockIdx.x & 7, qid = blockIdx.x >> 3;
-    const int ob = qid % a.n_oblk;
-    const int64_t strip_lin = (int64_t)(qid / a.n_oblk) * 8 + xcd;
-    if (strip_lin >= a.n_strips * a.B) return;
-    const int b = (int)(strip_lin / a.n_strips);
-    const int64_t pw0 = (strip_lin - (int64_t)b * a.n_strips) * DM_PX;
+    __shared__ __align__(16) unsigned char lds[DM_LDS];
+    // tiles of this XCD, row block fastest: q -> (row block q % n_oblk, strip (q / n_oblk) * 8 + xcd); the workgroups of the
+    // XCD deal them out round robin, so the row blocks of one strip run at the same time on one L2
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, nslot = gridDim.x >> 3;
+    const int strips = (int)(a.n_strips * a.B);
+    const int nq = xcd < strips ? (strips - xcd + 7) / 8 * a.n_oblk : 0;
+    if (slot >= nq) return;
+    const int ntl = (nq - slot + nslot - 1) / nslot;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wo = wave >> 1, wp = wave & 1;                    // 4 wavefronts along the rows x 2 along the pixels
     const int q = lane & 31, ko = lane >> 5;
-    const int o0 = ob * DM_ROWS + wo * 32 * DM_MT;
     const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)lds);
+    const bool wload = wave < 4;                                // this wavefront fetches weights (else activations)
+    const int lw = wave & 3;
 
-    // this wavefront's share of a chunk: weight blocks (k step wave >> 2, row blocks 3 (wave & 3) .. + 2) and
-    // activation blocks 2 wave, 2 wave + 1 (block = rows 2 xb, 2 xb + 1 of the chunk; lane = row (lane >> 5), 8 pixels (lane & 31))
     const int nc16 = a.Kpad / PW_KC;
     const int nchunks = a.Kpad / DM_CK;
-    const unsigned short* wsrc = a.W + (((int64_t)(ob * (DM_ROWS / 32) + 3 * (wave & 3)) * nc16 + (wave >> 2)) * 64 + lane) * 8;
     const int64_t wrb = (int64_t)nc16 * 512;                   // ushorts between row blocks
     // input channels k < K1 come from X, the others (if any) from X2: a convolution over the concatenation of two tensors
     const int K1 = a.X2 ? a.K1 : a.K;
-    const int64_t xpx = min(pw0 + 8 * (lane & 31), a.P - 8);
-    const unsigned short* __restrict__ X = a.X + (int64_t)b * K1 * a.P + xpx;
-    const unsigned short* __restrict__ X2 = a.X2 ? a.X2 + (int64_t)b * (a.K - K1) * a.P + xpx : X;
-    const int xrow0 = 4 * wave + (lane >> 5);                   // first of this lane's rows in the chunk: 2 (2 wave + i) + (lane >> 5)
 
-    auto issue = [&](int c, int stage) {
-        const unsigned sb = lds0 + stage * DM_STAGE;
-        const unsigned short* wp_ = wsrc + (int64_t)c * 1024;
-#pragma unroll
-        for (int i = 0; i < 3; ++i) dma16(wp_ + i * wrb, sb + ((wave >> 2) * 12 + 3 * (wave & 3) + i) * 1024);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int k = min(c * DM_CK + xrow0 + 2 * i, a.K - 1);      // rows past K meet zero weights
-            dma16(k < K1 ? X + (int64_t)k * a.P : X2 + (int64_t)(k - K1) * a.P, sb + DM_ABYTES + (2 * wave + i) * DM_XBLK);
+    const unsigned n_oblk = (unsigned)a.n_oblk, n_strips = (unsigned)a.n_strips;
+    auto tile_of = [&](int qq, int& ob, int& b, int64_t& pw0) {
+        const unsigned sl = (unsigned)qq / n_oblk * 8u + (unsigned)xcd;
+        ob = (int)((unsigned)qq % n_oblk);
+        b = (int)(sl / n_strips);
+        pw0 = (int64_t)(sl - (unsigned)b * n_strips) * DM_PX;
+    };
+
+    // load stream of this wavefront: weight blocks (row blocks 3 lw .. 3 lw + 2 of both 16-row k steps), or activation blocks
+    // 4 lw .. 4 lw + 3 (block xb = rows 2 xb, 2 xb + 1 of the chunk; lane = row (lane >> 5), 8 pixels (lane & 31))
+    int iq = slot, ic = 0, isg = 0;                             // next chunk to ask for: tile, chunk, stage
+    const unsigned short *sp0 = nullptr, *sp1 = nullptr;        // wavefront-uniform bases of the stream's tile
+    int voff = lane * 8;                                        // lane's offset from them, in elements
+    auto issue = [&]() -> bool {
+        if (iq >= nq) return false;
+        if (ic == 0) {
+            int ob, b;
+            int64_t pw0;
+            tile_of(iq, ob, b, pw0);
+            if (wload) {
+                sp0 = a.W + ((int64_t)(ob * (DM_ROWS / 32) + 3 * lw) * nc16) * 512;
+            } else {
+                sp0 = a.X + (int64_t)b * K1 * a.P;
+                sp1 = a.X2 ? a.X2 + (int64_t)b * (a.K - K1) * a.P : sp0;
+                voff = (int)min(pw0 + 8 * (lane & 31), a.P - 8);
+            }
         }
+        if (wload) {
+            const unsigned sb = lds0 + isg * DM_ABYTES + 3 * lw * 1024;
+            const unsigned short* src = sp0 + (int64_t)ic * 1024 + voff;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int i = 0; i < 3; ++i) dma16(src + ks * 512 + i * wrb, sb + (ks * 12 + i) * 1024);
+            isg = (isg == DM_WSTAGES - 1) ? 0 : isg + 1;
+        } else {
+            const unsigned sb = lds0 + DM_XBASE + isg * DM_XBYTES + 4 * lw * DM_XBLK;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // rows k0 and k0 + 1 for the two halves of the wavefront; rows past K meet zero weights
+                const int k0 = min(ic * DM_CK + 8 * lw + 2 * i, a.K - 1), k1 = min(k0 + 1, a.K - 1);
+                const unsigned short* r0 = k0 < K1 ? sp0 + (int64_t)k0 * a.P : sp1 + (int64_t)(k0 - K1) * a.P;
+                const unsigned short* r1 = k1 < K1 ? sp0 + (int64_t)k1 * a.P : sp1 + (int64_t)(k1 - K1) * a.P;
+                dma16((lane >> 5 ? r1 : r0) + voff, sb + i * DM_XBLK);
+            }
+            isg = (isg == DM_XSTAGES - 1) ? 0 : isg + 1;
+        }
+        if (++ic == nchunks) {
+            ic = 0;
+            iq += nslot;
+        }
+        return true;
     };
 
     f32x16 acc[DM_MT][DM_NT];
@@ -313,99 +370,184 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
 
-    issue(0, 0);
-    if (nchunks > 1) {
-        issue(1, 1);
-        __builtin_amdgcn_s_waitcnt(0x0F75);        // vmcnt(5): chunk 0 has landed
-    } else {
+    // fill the pipeline: three weight chunks or five activation chunks, then chunk 0 must have landed
+    bool full = true;
+    for (int i = 0; i < (wload ? DM_WSTAGES : DM_XSTAGES); ++i) full = issue() && full;
+    if (full)
+        __builtin_amdgcn_s_waitcnt(0x0F7C);        // vmcnt(12): two chunks of weights, three of the four later activation chunks
+    else
         __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
-    }
     __syncthreads();
 
     const unsigned char* abase = lds + (DM_MT * wo) * 1024 + lane * 16;
-    const unsigned char* xbase = lds + DM_ABYTES + (4 * ko) * DM_XBLK + wp * 256 + 8 * q;
-    int stage = 0;
-    for (int c = 0; c < nchunks; ++c) {
-        const int s2 = (stage == 0) ? 2 : stage - 1;            // (stage + 2) % 3
-        if (c + 2 < nchunks) issue(c + 2, s2);
-        const unsigned char* sa = abase + stage * DM_STAGE;
-        const unsigned char* sx = xbase + stage * DM_STAGE;
+    const unsigned char* xbase = lds + DM_XBASE + (4 * ko) * DM_XBLK + wp * 256 + 8 * q;
+    int sw = 0, sx = 0;
+    // Operands of a 16-row k step: eight raw words of activations (rw), regrouped by byte permutes into the four B fragments
+    // (bf), and three A fragments (af).  The LDS reads of the next k step are issued into rw and af as soon as the current
+    // step has consumed them (rw after the permutes, af[mt] after the MFMAs of row tile mt), so they run under the MFMAs.
+    u32x2 rw[8];
+    u32x4 af[DM_MT], bf[DM_NT];
+    auto load_rw = [&](const unsigned char* sxp, int ks) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            u32x2 rw[8];
+        for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const u32x2*>(sxp + (8 * ks + (r >> 1)) * DM_XBLK + (r & 1) * 512);
+    };
+    auto load_af = [&](const unsigned char* sa, int ks, int mt) { af[mt] = *reinterpret_cast<const u32x4*>(sa + (ks * 12 + mt) * 1024); };
+    auto regroup = [&]() {
 #pragma unroll
-            for (int r = 0; r < 8; ++r) rw[r] = *reinterpret_cast<const u32x2*>(sx + (8 * ks + (r >> 1)) * DM_XBLK + (r & 1) * 512);
-            u32x4 af[DM_MT];
+        for (int pp = 0; pp < 2; ++pp)
 #pragma unroll
-            for (int mt = 0; mt < DM_MT; ++mt) af[mt] = *reinterpret_cast<const u32x4*>(sa + (ks * 12 + mt) * 1024);
-            u32x4 bf[DM_NT];
+            for (int h = 0; h < 4; ++h) {
+                bf[2 * pp][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x05040100u);
+                bf[2 * pp + 1][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x07060302u);
+            }
+    };
+    auto mfma_row = [&](int mt) {
+        const bf16x8 av = __builtin_bit_cast(bf16x8, af[mt]);
 #pragma unroll
-            for (int pp = 0; pp < 2; ++pp)
+        for (int t = 0; t < DM_NT; ++t)
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+    };
+
+    // Epilogue of one tile, a quarter of a row tile (eight rows, of which a lane has the four of its half ko) at a time.
+    // Bias and the addend's scale and shift come through the scalar unit, the eight rows in one batch ahead of the four
+    // stores: a vector load between the stores would make each store wait for the one before, since the wait for the load
+    // covers every store issued before it.  The addend itself is read half a row tile ahead.
+    auto epilogue = [&](auto whole, int o0, int ko4, int b, int64_t lane_off) {
+        constexpr bool WHOLE = decltype(whole)::value;
+        unsigned short* __restrict__ Y = a.Y + lane_off;
+        const unsigned short* __restrict__ R = ADD ? a.addend + lane_off : nullptr;
+        auto row_of = [&](int mt, int v) { return 32 * mt + 8 * (v >> 2) + (v & 3); };     // without the lane's 4 ko
+        u32x2 rv[2][8];
+        auto load_addend = [&](int mh) {
+            if constexpr (ADD) {
 #pragma unroll
-                for (int h = 0; h < 4; ++h) {
-                    bf[2 * pp][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x05040100u);
-                    bf[2 * pp + 1][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x07060302u);
+                for (int j = 0; j < 8; ++j) {
+                    int r = row_of(mh >> 1, 8 * (mh & 1) + j);
+                    if (!WHOLE) r = min(r, a.O - 1 - o0 - ko4);
+                    rv[mh & 1][j] = *reinterpret_cast<const u32x2*>(R + (int64_t)r * a.P);
                 }
+            }
+        };
+        load_addend(0);
+#pragma unroll
+        for (int mh = 0; mh < 2 * DM_MT; ++mh) {
+            const int mt = mh >> 1;
+            if (!WHOLE && o0 + 32 * mt >= a.O) break;
+            if (mh + 1 < 2 * DM_MT && (WHOLE || o0 + 32 * ((mh + 1) >> 1) < a.O)) load_addend(mh + 1);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const int v0 = 8 * (mh & 1) + 4 * g;
+                const int oq = o0 + row_of(mt, v0);             // rows oq .. oq + 7 (ko = 0: oq .. oq + 3)
+                float ub[8], usc[8], ush[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int64_t u = WHOLE ? oq + i : min(oq + i, a.O - 1);
+                    ub[i] = a.bias ? uniform_load(a.bias, u) : 0.f;
+                    usc[i] = (ADD && a.add_scale) ? uniform_load(a.add_scale, (int64_t)b * a.O + u) : 1.f;
+                    ush[i] = (ADD && a.add_shift) ? uniform_load(a.add_shift, (int64_t)b * a.O + u) : 0.f;
+                }
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int v = v0 + jj;
+                    if (!WHOLE && oq + ko4 + jj >= a.O) continue;
+                    const float bs = ko4 ? ub[4 + jj] : ub[jj];
+                    float y[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) y[t] = acc[mt][t][v] + bs;
+                    if constexpr (GELU) {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) y[t] = gelu(y[t]);
+                    }
+                    if constexpr (ADD) {
+                        const float sc = ko4 ? usc[4 + jj] : usc[jj], sh = ko4 ? ush[4 + jj] : ush[jj];
+                        const u32x2 r = rv[mh & 1][4 * g + jj];
+#pragma unroll
+                        for (int pp = 0; pp < 2; ++pp) {
+                            y[2 * pp] += fmaf(sc, __uint_as_float(r[pp] << 16), sh);
+                            y[2 * pp + 1] += fmaf(sc, __uint_as_float(r[pp] & 0xffff0000u), sh);
+                        }
+                    }
+                    u32x2 out;
+#pragma unroll
+                    for (int pp = 0; pp < 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
+                    *reinterpret_cast<u32x2*>(Y + (int64_t)row_of(mt, v) * a.P) = out;
+                }
+            }
+        }
+    };
+
+    for (int tl = 0; tl < ntl; ++tl) {
+        const unsigned char* sa = abase + sw * DM_ABYTES;
+        const unsigned char* sxp = xbase + sx * DM_XBYTES;
+        load_rw(sxp, 0);
+#pragma unroll
+        for (int mt = 0; mt < DM_MT; ++mt) load_af(sa, 0, mt);
+        for (int c = 0; c < nchunks; ++c) {
+            // first k step of the chunk; the second one's operands follow it into the registers
+            regroup();
+            __builtin_amdgcn_sched_barrier(0);
+            load_rw(sxp, 1);
 #pragma unroll
             for (int mt = 0; mt < DM_MT; ++mt) {
-                const bf16x8 av = __builtin_bit_cast(bf16x8, af[mt]);
+                mfma_row(mt);
+                __builtin_amdgcn_sched_barrier(0);
+                load_af(sa, 1, mt);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            regroup();
+            // Every wavefront has read all of this chunk.  The next chunk must have landed for every wavefront before it is
+            // read; in flight may stay the loads of one weight chunk (6) or of three activation chunks (12), everything once
+            // the stream has run dry.  Then this chunk's stages take the chunk three (five) further on.
+            if (!full)
+                __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
+            else if (wload)
+                __builtin_amdgcn_s_waitcnt(0x0F76);    // vmcnt(6)
+            else
+                __builtin_amdgcn_s_waitcnt(0x0F7C);    // vmcnt(12)
+            __syncthreads();
+            full = issue();
+            sw = (sw == DM_WSTAGES - 1) ? 0 : sw + 1;
+            sx = (sx == DM_XSTAGES - 1) ? 0 : sx + 1;
+            sa = abase + sw * DM_ABYTES;
+            sxp = xbase + sx * DM_XBYTES;
+            // second k step; the first one of the next chunk follows (after the last chunk of a tile these reads are
+            // repeated behind the epilogue, which needs the registers)
+            __builtin_amdgcn_sched_barrier(0);
+            load_rw(sxp, 0);
 #pragma unroll
-                for (int t = 0; t < DM_NT; ++t)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+            for (int mt = 0; mt < DM_MT; ++mt) {
+                mfma_row(mt);
+                __builtin_amdgcn_sched_barrier(0);
+                load_af(sa, 0, mt);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // chunk c + 1 (issued one iteration ago) must have landed for every wavefront before it is read, and every
-        // wavefront must be done with this stage before chunk c + 3 overwrites it
-        if (c + 2 < nchunks)
-            __builtin_amdgcn_s_waitcnt(0x0F75);    // vmcnt(5): all but the loads of chunk c + 2
-        else
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        stage = (stage == 2) ? 0 : stage + 1;
-    }
 
-    // epilogue: lane holds rows 8 (v / 4) + 4 ko + v % 4 of each 32-row tile and pixels 4 q .. 4 q + 3
-    const int64_t px = pw0 + wp * 128 + 4 * q;
-    if (px >= a.P) return;
-    unsigned short* __restrict__ Y = a.Y + (int64_t)b * a.O * a.P;
-    const unsigned short* __restrict__ R = a.addend ? a.addend + (int64_t)b * a.O * a.P : nullptr;
-#pragma unroll
-    for (int mt = 0; mt < DM_MT; ++mt) {
-        if (o0 + 32 * mt >= a.O) break;
-        u32x2 rv[16];
-        if (R) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int o = min(o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3), a.O - 1);
-                rv[v] = *reinterpret_cast<const u32x2*>(R + (int64_t)o * a.P + px);
-            }
+        // epilogue: lane holds rows 8 (v / 4) + 4 ko + v % 4 of each 32-row tile and pixels 4 q .. 4 q + 3
+        int ob, b;
+        int64_t pw0;
+        tile_of(slot + tl * nslot, ob, b, pw0);
+        // (derived afresh for every tile: hoisted out of the tile loop, the row offsets of a lane and its addresses would
+        // occupy registers the accumulators need)
+        int lane_ = lane;
+        asm volatile("" : "+v"(lane_));
+        const int ko4 = (lane_ >> 5) * 4;
+        const int o0 = ob * DM_ROWS + wo * 32 * DM_MT;          // first row of the wavefront
+        const int64_t px = pw0 + wp * 128 + 4 * (lane_ & 31);
+        if (px < a.P && o0 < a.O) {
+            const int64_t lane_off = ((int64_t)b * a.O + o0 + ko4) * a.P + px;      // lane's first row
+            // whole wavefront tile inside the matrix: no row needs a check or a clamp
+            if (o0 + 32 * DM_MT <= a.O)
+                epilogue(std::true_type{}, o0, ko4, b, lane_off);
+            else
+                epilogue(std::false_type{}, o0, ko4, b, lane_off);
         }
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int o = o0 + 32 * mt + 8 * (v >> 2) + 4 * ko + (v & 3);
-            if (o >= a.O) continue;
-            const float bs = a.bias ? a.bias[o] : 0.f;
-            float y[4];
+        for (int mt = 0; mt < DM_MT; ++mt)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) y[t] = acc[mt][t][v] + bs;
-            if (a.act == SFNO_ACT_GELU) {
+            for (int t = 0; t < DM_NT; ++t)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) y[t] = gelu(y[t]);
-            }
-            if (R) {
-                const float sc = a.add_scale ? a.add_scale[(int64_t)b * a.O + o] : 1.f;
-                const float sh = a.add_shift ? a.add_shift[(int64_t)b * a.O + o] : 0.f;
-#pragma unroll
-                for (int pp = 0; pp < 2; ++pp) {
-                    y[2 * pp] += fmaf(sc, __uint_as_float(rv[v][pp] << 16), sh);
-                    y[2 * pp + 1] += fmaf(sc, __uint_as_float(rv[v][pp] & 0xffff0000u), sh);
-                }
-            }
-            u32x2 out;
-#pragma unroll
-            for (int pp = 0; pp < 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
-            *reinterpret_cast<u32x2*>(Y + (int64_t)o * a.P + px) = out;
-        }
+                for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
     }
 }
 
@@ -544,6 +686,17 @@ __global__ __launch_bounds__(256) void scale_shift_act_kernel(const unsigned sho
 
 }  // namespace
 
+// compute units of the current device (256 when the query fails)
+static int device_cus() {
+    static int cached[64] = {};
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
+    if (cached[dev] > 0) return cached[dev];
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) { (void)hipGetLastError(); return 256; }
+    cached[dev] = cus;
+    return cus;
+}
+
 int pointwise_kpad(int K) { return (K + PW_KALIGN - 1) / PW_KALIGN * PW_KALIGN; }
 // rows are padded to whole workgroup tiles so that no fragment load needs a bound check
 int pointwise_opad(int O) {
@@ -572,9 +725,16 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
     a.n_strips = (a.P + wpx - 1) / wpx;
     const int64_t strips = a.n_strips * a.B;
     const int64_t blocks = (strips + 7) / 8 * 8 * a.n_oblk;
-    if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    if (dma)
-        hipLaunchKernelGGL(pw_gemm_dma_kernel, dim3((unsigned)blocks), dim3(512), 0, s, a);
+    if (blocks > 0x7fffffffLL || (dma && a.P > 0x7fffffffLL)) return SFNO_EUNSUPPORTED;
+    if (dma)       // persistent: one workgroup per CU (its LDS admits no second one), the same number on every XCD
+    {
+        const dim3 grid((unsigned)std::min<int64_t>(blocks, std::max(8, device_cus() / 8 * 8)));
+        const bool g = a.act == SFNO_ACT_GELU, r = a.addend != nullptr;
+        if (g && r) hipLaunchKernelGGL((pw_gemm_dma_kernel<true, true>), grid, dim3(512), 0, s, a);
+        else if (g) hipLaunchKernelGGL((pw_gemm_dma_kernel<true, false>), grid, dim3(512), 0, s, a);
+        else if (r) hipLaunchKernelGGL((pw_gemm_dma_kernel<false, true>), grid, dim3(512), 0, s, a);
+        else hipLaunchKernelGGL((pw_gemm_dma_kernel<false, false>), grid, dim3(512), 0, s, a);
+    }
     else
         hipLaunchKernelGGL((pw_gemm_kernel<1, 2>), dim3((unsigned)blocks), dim3(512), 0, s, a);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;

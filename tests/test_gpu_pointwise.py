@@ -26,6 +26,10 @@ CONV_CASES = [
     (3, 73, 73, 9, 8, False, None, False, False),
     (1, 100, 200, 11, 24, True, "gelu", True, True),       # nothing a multiple of the tile sizes
     (1, 8, 5, 721, 1440, True, None, False, False),        # full-resolution grid, tiny channels
+    # several tiles per persistent workgroup (O > 96): the operand rings wrap and run on across tile boundaries
+    (1, 100, 500, 160, 1000, True, "gelu", True, True),    # two row blocks, the second partly filled; ragged last strip
+    (2, 73, 384, 125, 1000, False, None, False, False),    # four K chunks per tile, two samples
+    (1, 384, 200, 90, 1000, True, None, True, False),      # twelve K chunks per tile
 ]
 
 

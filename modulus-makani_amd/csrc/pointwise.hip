@@ -45,9 +45,10 @@ __device__ __forceinline__ float uniform_load(const float* p, int64_t i) {
 // exact (erf) GELU for bf16 outputs.  gelu(x) = max(x, 0) - |x| erfc(|x| / sqrt 2) / 2 for both signs (no cancellation in
 // the negative tail), and erfc is evaluated as 2^Q(|x|): log2 erfc(t / sqrt 2) is smooth, a degree-7 polynomial in t follows it
 // to 7e-5 on [0, 8.5] (relative error of erfc 5e-5, a fortieth of the half ulp of the bf16 result); beyond 8.5 the term is
-// below 1e-16 and t is clamped.  Eleven full-rate instructions and one exp2, where a rational form needs a reciprocal as well.
+// below 1e-16 and t is clamped.  Twelve full-rate instructions and one exp2, where a rational form needs a reciprocal as well.
 __device__ __forceinline__ float gelu(float x) {
-    const float t = fminf(fabsf(x), 8.5f);
+    // (the median of three stands for min and max: one instruction each, where fminf / fmaxf first canonicalise their operand)
+    const float t = __builtin_amdgcn_fmed3f(fabsf(x), 0.f, 8.5f);
     float q = fmaf(t, -1.112324808e-06f, 4.422128154e-05f);
     q = fmaf(t, q, -7.661478214e-04f);
     q = fmaf(t, q, 7.736902644e-03f);
@@ -55,7 +56,7 @@ __device__ __forceinline__ float gelu(float x) {
     q = fmaf(t, q, -4.605784664e-01f);
     q = fmaf(t, q, -1.150352355e+00f);
     q = fmaf(t, q, -5.705795628e-05f);
-    return fmaf(-0.5f * fabsf(x), __builtin_amdgcn_exp2f(q), fmaxf(x, 0.f));
+    return fmaf(-0.5f * fabsf(x), __builtin_amdgcn_exp2f(q), __builtin_amdgcn_fmed3f(x, 0.f, __builtin_inff()));
 }
 
 // WM = wavefronts along the output rows: 4 (x 2 along pixels: 384 rows x 128 pixels per workgroup) or

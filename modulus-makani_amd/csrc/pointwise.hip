@@ -429,7 +429,21 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
                 }
             }
         };
+        // scalar loads one quarter ahead: those of quarter q + 1 are issued once those of quarter q have arrived (the wait of the
+        // scalar unit is for all of its loads at once), and are under way while quarter q is converted and stored
+        float ub[2][8], usc[2][8], ush[2][8];
+        auto load_scalars = [&](int qq) {
+            const int oq = o0 + row_of(qq >> 2, 4 * (qq & 3));   // rows oq .. oq + 7 (ko = 0: oq .. oq + 3)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t u = WHOLE ? oq + i : min(oq + i, a.O - 1);
+                ub[qq & 1][i] = a.bias ? uniform_load(a.bias, u) : 0.f;
+                usc[qq & 1][i] = (ADD && a.add_scale) ? uniform_load(a.add_scale, (int64_t)b * a.O + u) : 1.f;
+                ush[qq & 1][i] = (ADD && a.add_shift) ? uniform_load(a.add_shift, (int64_t)b * a.O + u) : 0.f;
+            }
+        };
         load_addend(0);
+        load_scalars(0);
 #pragma unroll
         for (int mh = 0; mh < 2 * DM_MT; ++mh) {
             const int mt = mh >> 1;
@@ -437,21 +451,18 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
             if (mh + 1 < 2 * DM_MT && (WHOLE || o0 + 32 * ((mh + 1) >> 1) < a.O)) load_addend(mh + 1);
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
+                const int qq = 2 * mh + g;
                 const int v0 = 8 * (mh & 1) + 4 * g;
-                const int oq = o0 + row_of(mt, v0);             // rows oq .. oq + 7 (ko = 0: oq .. oq + 3)
-                float ub[8], usc[8], ush[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int64_t u = WHOLE ? oq + i : min(oq + i, a.O - 1);
-                    ub[i] = a.bias ? uniform_load(a.bias, u) : 0.f;
-                    usc[i] = (ADD && a.add_scale) ? uniform_load(a.add_scale, (int64_t)b * a.O + u) : 1.f;
-                    ush[i] = (ADD && a.add_shift) ? uniform_load(a.add_shift, (int64_t)b * a.O + u) : 0.f;
-                }
+                const int oq = o0 + row_of(mt, v0);
+                asm volatile("" ::"s"(ub[qq & 1][0]), "s"(ub[qq & 1][7]));       // the wait for this quarter's scalars goes here
+                __builtin_amdgcn_sched_barrier(0);
+                if (qq + 1 < 4 * DM_MT) load_scalars(qq + 1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) {
                     const int v = v0 + jj;
                     if (!WHOLE && oq + ko4 + jj >= a.O) continue;
-                    const float bs = ko4 ? ub[4 + jj] : ub[jj];
+                    const float bs = ko4 ? ub[qq & 1][4 + jj] : ub[qq & 1][jj];
                     float y[4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) y[t] = acc[mt][t][v] + bs;
@@ -460,7 +471,7 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
                         for (int t = 0; t < 4; ++t) y[t] = gelu(y[t]);
                     }
                     if constexpr (ADD) {
-                        const float sc = ko4 ? usc[4 + jj] : usc[jj], sh = ko4 ? ush[4 + jj] : ush[jj];
+                        const float sc = ko4 ? usc[qq & 1][4 + jj] : usc[qq & 1][jj], sh = ko4 ? ush[qq & 1][4 + jj] : ush[qq & 1][jj];
                         const u32x2 r = rv[mh & 1][4 * g + jj];
 #pragma unroll
                         for (int pp = 0; pp < 2; ++pp) {

@@ -364,12 +364,6 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
     };
 
     f32x16 acc[DM_MT][DM_NT];
-#pragma unroll
-    for (int mt = 0; mt < DM_MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < DM_NT; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
 
     // fill the pipeline: three weight chunks or five activation chunks, then chunk 0 must have landed
     bool full = true;
@@ -402,11 +396,19 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
                 bf[2 * pp + 1][h] = __builtin_amdgcn_perm(rw[2 * h + 1][pp], rw[2 * h][pp], 0x07060302u);
             }
     };
-    auto mfma_row = [&](int mt) {
+    // (the first k step of a tile starts its sums from the constant zero: no pass over the 192 accumulators between tiles)
+    auto mfma_row = [&](int mt, bool first) {
         const bf16x8 av = __builtin_bit_cast(bf16x8, af[mt]);
+        if (first) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < DM_NT; ++t)
-            acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+            for (int t = 0; t < DM_NT; ++t)
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), zero, 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int t = 0; t < DM_NT; ++t)
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, bf[t]), acc[mt][t], 0, 0, 0);
+        }
     };
 
     // Epilogue of one tile, a quarter of a row tile (eight rows, of which a lane has the four of its half ko) at a time.
@@ -501,7 +503,7 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
             load_rw(sxp, 1);
 #pragma unroll
             for (int mt = 0; mt < DM_MT; ++mt) {
-                mfma_row(mt);
+                mfma_row(mt, c == 0);
                 __builtin_amdgcn_sched_barrier(0);
                 load_af(sa, 1, mt);
                 __builtin_amdgcn_sched_barrier(0);
@@ -528,7 +530,7 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
             load_rw(sxp, 0);
 #pragma unroll
             for (int mt = 0; mt < DM_MT; ++mt) {
-                mfma_row(mt);
+                mfma_row(mt, false);
                 __builtin_amdgcn_sched_barrier(0);
                 load_af(sa, 0, mt);
                 __builtin_amdgcn_sched_barrier(0);
@@ -554,12 +556,6 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
             else
                 epilogue(std::false_type{}, o0, ko4, b, lane_off);
         }
-#pragma unroll
-        for (int mt = 0; mt < DM_MT; ++mt)
-#pragma unroll
-            for (int t = 0; t < DM_NT; ++t)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[mt][t][v] = 0.f;
     }
 }
 

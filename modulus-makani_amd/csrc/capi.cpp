@@ -550,7 +550,7 @@ extern "C" int sfno_diagonal_weight_grad(const void* x, const void* gy, void* gw
 
 extern "C" int64_t sfno_pointwise_weight_elems(int O, int K) {
     if (O < 1 || K < 1) return 0;
-    return (int64_t)pointwise_opad(O) * pointwise_kpad(K);
+    return (int64_t)pointwise_opad(O) * pointwise_kpad(K, O);
 }
 
 extern "C" int sfno_pointwise_pack_weight(const float* w, void* packed, int O, int K, void* stream) {

@@ -261,8 +261,9 @@ __global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseA
 // next tile are already in LDS when the stores of the current one leave.  A read only reaches the HBM rate with
 // some 50 KB in flight per CU, and the memory counter of a wavefront retires in order, so a wavefront that waits for
 // a weight block (an L2 hit) would also wait for every activation block it asked for earlier.  The two streams
-// therefore belong to different wavefronts: wavefronts 0-3 fetch the weights two chunks ahead (three stages of
-// 24 KiB), wavefronts 4-7 the activations four chunks ahead (five stages of 16 KiB: 64 KiB in flight).  The loads are
+// therefore belong to different wavefronts: wavefronts 0-3 fetch the weights into three stages of 24 KiB, wavefronts
+// 4-7 the activations into five stages of 16 KiB; a stage is asked for again as soon as every wavefront has read it, so
+// two to three weight chunks and four to five activation chunks (64-80 KiB) are on their way or waiting.  The loads are
 // issued from inline assembly (the compiler would order every LDS read behind all outstanding direct-to-LDS loads)
 // and the waits are written out by hand.  Other memory operations of a wavefront (the epilogue's stores and addend
 // loads) are older than the loads a wait is meant for or younger than all of them; either way the wait covers
@@ -274,7 +275,7 @@ constexpr int DM_CK = 32;                        // k rows per chunk
 constexpr int DM_ABYTES = 2 * (DM_ROWS / 32) * 1024;   // weight stage: 24 fragment blocks of 1 KiB
 constexpr int DM_XBLK = 1024 + 16;               // two pixel rows of the chunk (2 x 512 bytes) + padding
 constexpr int DM_XBYTES = (DM_CK / 2) * DM_XBLK; // activation stage
-constexpr int DM_WSTAGES = 3, DM_XSTAGES = 5;    // prefetch distance + 1
+constexpr int DM_WSTAGES = 3, DM_XSTAGES = 5;    // chunks in LDS or on their way, per stream
 constexpr int DM_XBASE = DM_WSTAGES * DM_ABYTES;
 constexpr int DM_LDS = DM_XBASE + DM_XSTAGES * DM_XBYTES;
 static_assert(DM_LDS <= 160 * 1024, "one workgroup per CU");
@@ -705,7 +706,11 @@ static int device_cus() {
     return cus;
 }
 
-int pointwise_kpad(int K) { return (K + PW_KALIGN - 1) / PW_KALIGN * PW_KALIGN; }
+// the kernel for O > 96 walks K in chunks of 32 rows and takes any number of them; the other one runs whole unrolled loop bodies
+int pointwise_kpad(int K, int O) {
+    const int align = O > PW_ROWS ? DM_CK : PW_KALIGN;
+    return (K + align - 1) / align * align;
+}
 // rows are padded to whole workgroup tiles so that no fragment load needs a bound check
 int pointwise_opad(int O) {
     const int tile = O > PW_ROWS ? 4 * PW_ROWS : PW_ROWS;
@@ -713,7 +718,7 @@ int pointwise_opad(int O) {
 }
 
 int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, hipStream_t s) {
-    const int nc = pointwise_kpad(K) / PW_KC;
+    const int nc = pointwise_kpad(K, O) / PW_KC;
     const int64_t total = (int64_t)(pointwise_opad(O) / 32) * nc * 512;
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
@@ -722,7 +727,7 @@ int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, 
 }
 
 int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s) {
-    a.Kpad = pointwise_kpad(a.K);
+    a.Kpad = pointwise_kpad(a.K, a.O);
     if (a.P % 8 != 0 || a.K < 1 || a.O < 1 || a.B < 1 || a.P < 8) return SFNO_EUNSUPPORTED;
     const bool tall = a.O > PW_ROWS;              // several wavefronts share a pixel strip
     const int wm = tall ? 4 : 1;

@@ -88,7 +88,7 @@ struct PointwiseArgs {
     int64_t n_strips;
 };
 int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s);
-int pointwise_kpad(int K);
+int pointwise_kpad(int K, int O);
 int pointwise_opad(int O);
 int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, hipStream_t s);
 int row_stats_segments(int64_t rows, int64_t P);

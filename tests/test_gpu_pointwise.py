@@ -21,7 +21,7 @@ CONV_CASES = [
     (2, 384, 768, 16, 24, True, "gelu", False, False),     # MLP fc1
     (1, 768, 384, 16, 24, True, None, False, False),       # MLP fc2
     (2, 384, 384, 13, 8, False, None, True, True),         # outer skip + norm1(y); strip shorter than a tile
-    (1, 73, 384, 20, 36, True, "gelu", False, False),      # encoder fc1: K padded 73 -> 128
+    (1, 73, 384, 20, 36, True, "gelu", False, False),      # encoder fc1: K padded 73 -> 96
     (1, 384, 73, 20, 36, False, None, True, False),        # decoder fc2 + big skip (O < 96: four wavefronts along pixels)
     (3, 73, 73, 9, 8, False, None, False, False),
     (1, 100, 200, 11, 24, True, "gelu", True, True),       # nothing a multiple of the tile sizes

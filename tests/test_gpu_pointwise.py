@@ -228,7 +228,8 @@ def test_conv1x1_over_two_tensors(lib_built):
     from makani_amd import pointwise as pw
 
     g = torch.Generator().manual_seed(21)
-    for (B, K1, K2, O, H, W) in ((1, 384, 384, 384, 24, 40), (2, 50, 77, 128, 16, 24), (1, 32, 416, 200, 8, 64), (2, 384, 73, 73, 16, 40), (1, 5, 3, 7, 8, 8)):
+    for (B, K1, K2, O, H, W) in ((1, 384, 384, 384, 24, 40), (2, 50, 77, 128, 16, 24), (1, 32, 416, 200, 8, 64), (2, 384, 73, 73, 16, 40), (1, 5, 3, 7, 8, 8),
+                                 (1, 73, 100, 200, 125, 1000)):     # several tiles per persistent workgroup, odd K1
         x1 = torch.randn(B, K1, H, W, generator=g).bfloat16().cuda()
         x2 = torch.randn(B, K2, H, W, generator=g).bfloat16().cuda()
         w = (torch.randn(O, K1 + K2, generator=g) / (K1 + K2) ** 0.5).cuda()

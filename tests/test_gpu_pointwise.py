@@ -30,6 +30,7 @@ CONV_CASES = [
     (1, 100, 500, 160, 1000, True, "gelu", True, True),    # two row blocks, the second partly filled; ragged last strip
     (2, 73, 384, 125, 1000, False, None, False, False),    # four K chunks per tile, two samples
     (1, 384, 200, 90, 1000, True, None, True, False),      # twelve K chunks per tile
+    (2, 128, 200, 123, 1000, True, "gelu", True, True),    # ragged last strip of every sample, several tiles per workgroup
 ]
 
 

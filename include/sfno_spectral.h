@@ -71,14 +71,17 @@ extern "C" {
 #define SFNO_DTYPE_BF16 1
 
 /* arithmetic of the Legendre / channel-mix contractions */
-#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  The Legendre stage and the channel mix run them on
-                                  * the bf16 matrix pipe: each operand is cut exactly into three bf16 numbers and the
-                                  * six products larger than 2^-23 of the result are accumulated in fp32 (error of the
-                                  * size of fp32 rounding).  Channel mixes with an odd number of input channels run
-                                  * on fp32 MFMA. */
+#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  The channel mix runs them on the fp16 matrix pipe: each
+                                  * operand row is scaled by a power of two and cut into two fp16 numbers (22 of its 24
+                                  * significant bits), three products per term are accumulated in fp32 and the scales are
+                                  * undone on output (error of the size of fp32 rounding, relative to |x||w| summed
+                                  * over the row).  The Legendre stage uses three exact bf16 parts per operand and six
+                                  * products.  Channel mixes with an odd number of input channels run on fp32 MFMA. */
 #define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs (tables and activations rounded to bf16), fp32 accumulate */
 #define SFNO_COMPUTE_FP32_MFMA 2 /* transform plans only: as SFNO_COMPUTE_FP32 with the Legendre stage on the fp32 MFMA
                                   * instruction (fp32 tables, no operand splitting) */
+#define SFNO_COMPUTE_FP32_BF16X3 3 /* as SFNO_COMPUTE_FP32 with every operand cut exactly into three bf16 numbers and the six
+                                  * products larger than 2^-23 of the result accumulated in fp32 (no scales) */
 
 /* activation fused into the pointwise kernels */
 #define SFNO_ACT_NONE 0

@@ -409,17 +409,28 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
     if (!out) return SFNO_EINVAL;
     *out = nullptr;
     if (I < 1 || O < 1 || L < 1) return SFNO_EINVAL;
-    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16) return SFNO_EUNSUPPORTED;
+    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16 && compute != SFNO_COMPUTE_FP32_BF16X3) return SFNO_EUNSUPPORTED;
     // the bf16 kernel reads activation rows in groups of four floats
     if (compute == SFNO_COMPUTE_BF16 && (2 * I) % 4 != 0) return SFNO_EUNSUPPORTED;
     sfno_dhconv_weights* w = new (std::nothrow) sfno_dhconv_weights();
     if (!w) return SFNO_ENOMEM;
     w->I = I; w->O = O; w->L = L; w->compute = compute;
     // fp32 on the bf16 matrix pipe reads activation rows in groups of four floats; odd channel counts stay on fp32 MFMA
-    w->split = compute == SFNO_COMPUTE_FP32 && (2 * I) % 4 == 0;
+    w->split = compute == SFNO_COMPUTE_FP32_BF16X3 && (2 * I) % 4 == 0;
+    w->f16 = compute == SFNO_COMPUTE_FP32 && (2 * I) % 4 == 0;
     if (hipGetDevice(&w->device) != hipSuccess) { delete w; return SFNO_EHIP; }
     size_t bytes;
-    if (w->split) {
+    if (w->f16) {
+        const int co = 32 * dhconv_f16_ntc(O);              // output channels per column block
+        w->nob = (O + co - 1) / co;
+        w->nc = (I + 15) / 16;
+        bytes = (size_t)128 * co * L * w->nob * w->nc;      // (Re, Im) x 2 planes x co x 16 complex fp16 per (degree, column block, chunk)
+        if (hipMalloc((void**)&w->d_cinv, sizeof(float) * co * (size_t)L * w->nob) != hipSuccess ||
+            hipMalloc((void**)&w->d_cmax, sizeof(float) * (size_t)L * O) != hipSuccess) {
+            sfno_dhconv_weights_destroy(w);
+            return SFNO_ENOMEM;
+        }
+    } else if (w->split) {
         w->nob = (2 * O + 127) / 128;
         w->nc = (2 * I + 15) / 16;
         bytes = 6144 * (size_t)L * w->nob * w->nc;          // 3 planes x 64 x 8 complex bf16 per (degree, column block, chunk)
@@ -432,13 +443,16 @@ extern "C" int sfno_dhconv_weights_create(int I, int O, int L, int compute, sfno
         w->nc = (2 * I + PG_KC - 1) / PG_KC;
         bytes = sizeof(float) * 1024 * (size_t)L * w->nob * w->nc;   // 8 x 64 complex fp32
     }
-    if (hipMalloc((void**)&w->d_W, bytes) != hipSuccess) { delete w; return SFNO_ENOMEM; }
+    if (hipMalloc((void**)&w->d_W, bytes) != hipSuccess) { sfno_dhconv_weights_destroy(w); return SFNO_ENOMEM; }
     *out = w;
     return SFNO_OK;
 }
 
 static int pack_weights(sfno_dhconv_weights* w, const void* weight, int adjoint, void* stream) {
     if (!w || !weight) return SFNO_EINVAL;
+    if (w->f16)
+        return dhconv_pack_f16_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->d_cinv, w->d_cmax, w->I, w->O, w->L, adjoint,
+                                      (hipStream_t)stream);
     if (w->split)
         return dhconv_pack_split_launch(reinterpret_cast<const float2*>(weight), w->d_W, w->I, w->O, w->L, adjoint, (hipStream_t)stream);
     if (w->compute == SFNO_COMPUTE_BF16)
@@ -471,6 +485,8 @@ extern "C" int sfno_dhconv_weight_grad(int I, int O, int L, const float* spec_in
 extern "C" int sfno_dhconv_weights_destroy(sfno_dhconv_weights* w) {
     if (!w) return SFNO_OK;
     if (w->d_W) (void)hipFree(w->d_W);
+    if (w->d_cinv) (void)hipFree(w->d_cinv);
+    if (w->d_cmax) (void)hipFree(w->d_cmax);
     delete w;
     return SFNO_OK;
 }
@@ -492,6 +508,8 @@ extern "C" int sfno_dhconv_spectral(const sfno_dhconv_weights* w, const float* s
     a.ld_out = (int)sfno_spectral_ld((int64_t)batch * w->O);
     a.nob = w->nob;
     a.nc = w->nc;
+    a.cinv = w->d_cinv;
+    if (w->f16) return dhconv_f16_launch(a, (hipStream_t)stream);
     if (w->split) return dhconv_split_launch(a, (hipStream_t)stream);
     if (w->compute == SFNO_COMPUTE_BF16) return dhconv_bf16_launch(a, (hipStream_t)stream);
     return dhconv_launch(a, (hipStream_t)stream);

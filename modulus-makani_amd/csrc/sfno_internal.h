@@ -47,6 +47,7 @@ struct DhconvArgs {
     float* Y;                      // spectral layout, rows of 2*O floats
     int B, I2, O2, L, M, tri, ld_in, ld_out;
     int nob, nc;                   // column blocks of DH_COLS over 2*O, K chunks of 16 over 2*I
+    const float* cinv;             // fp16-pair kernel: [L][nob * channels per block] factors that undo the column scales of the packed weights
 };
 int dhconv_launch(const DhconvArgs& a, hipStream_t s);
 // bf16 MFMA variant: 256 output columns per workgroup, K chunks of 32, weights packed as complex bf16
@@ -55,6 +56,12 @@ int dhconv_bf16_launch(const DhconvArgs& a, hipStream_t s);
 // complex bf16 whose sum is the fp32 weight
 int dhconv_split_launch(const DhconvArgs& a, hipStream_t s);
 int dhconv_pack_split_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s);
+// fp32 operands on the fp16 matrix pipe (two fp16 planes per operand, power-of-two scales per weight column and per activation
+// row): 32 dhconv_f16_ntc(O) output channels per workgroup (a.nob blocks of them), a.nc chunks of 16 input channels; cinv
+// receives [L][nob * 32 ntc] inverse column scales, cmax is [L][O] scratch
+int dhconv_f16_ntc(int O);
+int dhconv_f16_launch(const DhconvArgs& a, hipStream_t s);
+int dhconv_pack_f16_launch(const float2* w, void* packed, float* cinv, float* cmax, int I, int O, int L, int adjoint, hipStream_t s);
 // adjoint = 1 packs the conjugate transpose: w then has shape [O][I][L] and element (i, o) is conj(w[o][i])
 int dhconv_pack_bf16_launch(const float2* w, void* packed, int I, int O, int L, int adjoint, hipStream_t s);
 // gradient of the contraction with respect to its weight:
@@ -194,6 +201,9 @@ struct sfno_sht_plan {
 struct sfno_dhconv_weights {
     int I, O, L, compute, device;
     int split;                     // fp32 compute with the weights stored as three bf16 planes (even in_channels)
+    int f16;                       // fp32 compute with the weights stored as two scaled fp16 planes (even in_channels)
     int nob, nc;                   // column blocks (over 2*O) and K chunks (over 2*I) per degree
     float* d_W = nullptr;          // packed complex weights
+    float* d_cinv = nullptr;       // f16: [L][nob * channels per block] inverse column scales
+    float* d_cmax = nullptr;       // f16: [L][O] scratch of the pack kernels
 };

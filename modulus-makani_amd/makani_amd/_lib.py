@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libsfno_spectral.so")
 GRID = {"legendre-gauss": 0, "lobatto": 1, "equiangular": 2, "planar": 3}
 NORM = {"ortho": 0, "four-pi": 1, "schmidt": 2}
 DIR_FORWARD, DIR_INVERSE, DIR_FORWARD_ADJOINT, DIR_INVERSE_ADJOINT = 1, 2, 4, 8
-COMPUTE_FP32, COMPUTE_BF16, COMPUTE_FP32_MFMA = 0, 1, 2
+COMPUTE_FP32, COMPUTE_BF16, COMPUTE_FP32_MFMA, COMPUTE_FP32_BF16X3 = 0, 1, 2, 3
 DTYPE_F32, DTYPE_BF16 = 0, 1
 ACT_NONE, ACT_GELU = 0, 1
 

@@ -50,7 +50,7 @@ class PackedWeights:
 
 
 # arithmetic of the contraction: fp32 MFMA, or bf16 MFMA inputs with fp32 accumulation
-COMPUTE = {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16}
+COMPUTE = {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16, "fp32_bf16x3": _lib.COMPUTE_FP32_BF16X3}
 
 # (id(tensor), compute) -> (weak reference to the tensor, PackedWeights); tensors compare element-wise,
 # so they cannot key a WeakKeyDictionary directly
@@ -63,7 +63,7 @@ def packed_for(weight, compute="fp32", adjoint=False):
     if weight.device.type != "cuda":
         raise RuntimeError("the dhconv kernel runs on a HIP device only")
     if compute not in COMPUTE:
-        raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32' or 'bf16'")
+        raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32', 'fp32_bf16x3' or 'bf16'")
     key = (id(weight), compute, adjoint)
     shape = (weight.shape[1], weight.shape[0], weight.shape[2]) if adjoint else tuple(weight.shape)
     hit = _cache.get(key)

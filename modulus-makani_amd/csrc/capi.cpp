@@ -25,6 +25,7 @@ int upload(T** dst, const std::vector<T>& src) {
 
 void free_table(PgemmTable& t) {
     if (t.d_A) (void)hipFree(t.d_A);
+    if (t.d_rinv) (void)hipFree(t.d_rinv);
     if (t.d_aoff) (void)hipFree(t.d_aoff);
     if (t.d_work) (void)hipFree(t.d_work);
     t = PgemmTable();
@@ -37,7 +38,8 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     std::vector<float> packed;
     std::vector<int64_t> aoff;
     std::vector<double> kept;          // mean number of K chunks a row block of order m runs through
-    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.format, packed, aoff, &kept);
+    std::vector<float> rinv;
+    pack_legendre_fold(gen, lat_w, order_scale, analysis, p.format, packed, aoff, &kept, &rinv);
     // a workgroup covers two 32-row blocks of each parity
     const int K2 = (p.nlat + 1) / 2;
     std::vector<int> nrb(p.mmax);
@@ -57,6 +59,7 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     t.n_blocks = (int64_t)(packed.size() / pg_block_floats(p.format));
     int rc;
     if ((rc = upload(&t.d_A, packed)) != SFNO_OK) return rc;
+    if (p.format == PG_FORMAT_F16X2 && (rc = upload(&t.d_rinv, rinv)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_aoff, aoff)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_work, work)) != SFNO_OK) return rc;
     return SFNO_OK;
@@ -87,6 +90,7 @@ PgemmArgs legendre_args(const sfno_sht_plan* p, const PgemmTable& t, const float
     a.work = t.d_work;
     a.Q = q;
     a.Out = out;
+    a.rinv = t.d_rinv;
     a.lmax = p->lmax;
     a.nlat = p->nlat;
     a.mmax = p->mmax;
@@ -171,14 +175,16 @@ extern "C" int sfno_sht_plan_create(int nlat, int nlon, int lmax, int mmax, int 
     if (grid < 0 || grid > SFNO_GRID_PLANAR || norm < 0 || norm > 2) return SFNO_EINVAL;
     if (grid == SFNO_GRID_PLANAR && (lmax > nlat || mmax > nlon / 2 + 1)) return SFNO_EINVAL;
     if (!(directions & all_dirs) || (directions & ~all_dirs)) return SFNO_EINVAL;
-    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16 && compute != SFNO_COMPUTE_FP32_MFMA) return SFNO_EUNSUPPORTED;
+    if (compute != SFNO_COMPUTE_FP32 && compute != SFNO_COMPUTE_BF16 && compute != SFNO_COMPUTE_FP32_MFMA && compute != SFNO_COMPUTE_FP32_BF16X3)
+        return SFNO_EUNSUPPORTED;
     sfno_sht_plan* p = new (std::nothrow) sfno_sht_plan();
     if (!p) return SFNO_ENOMEM;
     p->nlat = nlat; p->nlon = nlon; p->lmax = lmax; p->mmax = mmax;
     p->grid = grid; p->norm = norm; p->csphase = csphase ? 1 : 0;
     p->directions = directions;
     p->compute = compute == SFNO_COMPUTE_BF16 ? SFNO_COMPUTE_BF16 : SFNO_COMPUTE_FP32;
-    p->format = compute == SFNO_COMPUTE_BF16 ? PG_FORMAT_BF16 : compute == SFNO_COMPUTE_FP32_MFMA ? PG_FORMAT_FP32 : PG_FORMAT_SPLIT;
+    p->format = compute == SFNO_COMPUTE_BF16 ? PG_FORMAT_BF16 : compute == SFNO_COMPUTE_FP32_MFMA ? PG_FORMAT_FP32
+                : compute == SFNO_COMPUTE_FP32_BF16X3 ? PG_FORMAT_SPLIT : PG_FORMAT_F16X2;
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return SFNO_EHIP; }
     // set-up of sfno_sht_forward_static on this device; a failure is reported by that entry point, not here
     (void)static_scratch_prepare();

@@ -335,6 +335,7 @@ static int launch_fold(const PgemmArgs& a, int n_work, hipStream_t s) {
 
 int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_work, hipStream_t s) {
     switch (format) {
+        case PG_FORMAT_F16X2: return legendre_f16_launch(analysis, a, n_work, s);
         case PG_FORMAT_BF16: return analysis ? launch_fold<true, LF_BF16>(a, n_work, s) : launch_fold<false, LF_BF16>(a, n_work, s);
         case PG_FORMAT_SPLIT: return analysis ? launch_fold<true, LF_SPLIT>(a, n_work, s) : launch_fold<false, LF_SPLIT>(a, n_work, s);
         case PG_FORMAT_FP32: return analysis ? launch_fold<true, LF_FP32>(a, n_work, s) : launch_fold<false, LF_FP32>(a, n_work, s);

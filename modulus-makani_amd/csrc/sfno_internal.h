@@ -23,6 +23,7 @@ constexpr int PG_WAVES = 4;        // wavefronts (= row blocks) per workgroup
 
 struct PgemmTable {
     float* d_A = nullptr;          // packed stream
+    float* d_rinv = nullptr;       // two-part fp16 format: 32 factors per row-block entry that undo the row scales
     int64_t* d_aoff = nullptr;     // index of the stream, see pack_legendre_fold
     int2* d_work = nullptr;        // [n_work] {batch, first row block} per workgroup, -1 = idle
     int n_work = 0;                // multiple of 8 (one queue per XCD, interleaved)
@@ -35,6 +36,7 @@ struct PgemmArgs {
     const int2* work;
     const float* Q;
     float* Out;
+    const float* rinv;             // two-part fp16 format: row factors, [entry position - 2 mmax][32]
     int lmax, nlat, mmax;          // Legendre modes
     int ld;                        // channel leading dimension of Q and Out (Legendre modes)
 };
@@ -124,15 +126,20 @@ void build_worklist(const std::vector<int>& nrb, const std::vector<double>& cost
 //   PG_FORMAT_FP32 : 512 floats, fragments of v_mfma_f32_32x32x2_f32
 //   PG_FORMAT_BF16 : 8 bf16 per lane (rounded to nearest even), 256 floats = 1 KiB
 //   PG_FORMAT_SPLIT: three planes of 8 bf16 per lane whose sum is the fp32 value exactly, 768 floats = 3 KiB
-enum { PG_FORMAT_FP32 = 0, PG_FORMAT_BF16 = 1, PG_FORMAT_SPLIT = 2 };
+//   PG_FORMAT_F16X2: two planes of 8 fp16 per lane, the entry times a power of two per row (rounded, and the rounded remainder),
+//                    512 floats = 2 KiB; the factors that undo the row scales go to a separate array
+enum { PG_FORMAT_FP32 = 0, PG_FORMAT_BF16 = 1, PG_FORMAT_SPLIT = 2, PG_FORMAT_F16X2 = 3 };
 inline int pg_block_floats(int format) { return format == PG_FORMAT_BF16 ? 256 : format == PG_FORMAT_SPLIT ? 768 : 512; }
 // value = P * lat_w[k] * order_scale[m]; a null pointer stands for all ones
 // aoff: [2 m + p] -> position in aoff of the stream's first row-block entry; entry of row block rb (at that position + rb) =
 // first block of the row block | (number of leading K chunks left out as negligible << 48); chunks_per_rb (optional): mean
 // number of kept chunks per row block of every order (work-list cost)
+// rinv (PG_FORMAT_F16X2): 32 row factors per row-block entry, in the order of the entries
 void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
-                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb = nullptr);
+                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb = nullptr,
+                        std::vector<float>* rinv = nullptr);
 int legendre_fold_launch(bool analysis, int format, const PgemmArgs& a, int n_work, hipStream_t s);
+int legendre_f16_launch(bool analysis, const PgemmArgs& a, int n_work, hipStream_t s);
 
 // ---- FFT (fft.hip) -----------------------------------------------------------------------
 struct FftPlan {

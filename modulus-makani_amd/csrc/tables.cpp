@@ -230,13 +230,46 @@ static void pack_block_split(unsigned short* blk, int rb, int c, int rows, int K
         }
 }
 
+// fp16 with round-to-nearest-even from a double (|v| below 65520); returns the bits and the rounded value
+static unsigned short f16_rne(double v, double* rounded) {
+    const unsigned short sign = std::signbit(v) ? 0x8000u : 0u;
+    const double av = std::fabs(v);
+    int e = 0;
+    if (av != 0.0) (void)std::frexp(av, &e);
+    const int E = std::max(e - 1, -14);                       // binade of the value (subnormals share the lowest one)
+    const double q = std::ldexp(1.0, E - 10);                 // spacing of fp16 numbers there
+    const double r = std::nearbyint(av / q) * q;              // ties to even (default rounding mode)
+    if (rounded) *rounded = sign ? -r : r;
+    if (r == 0.0) return sign;
+    int e2;
+    const double f2 = std::frexp(r, &e2);                     // r = f2 * 2^e2, f2 in [0.5, 1)
+    if (e2 - 1 < -14) return (unsigned short)(sign | (unsigned)std::lround(std::ldexp(r, 24)));
+    return (unsigned short)(sign | ((unsigned)(e2 - 1 + 15) << 10) | ((unsigned)std::lround(std::ldexp(f2, 11)) - 1024u));
+}
+
+// two-part fp16 flavour: block = 2 planes x 64 lanes x 8 fp16, same (lane, e) -> (row, k) map as the bf16 flavour; plane 0
+// holds the entry times 2^sh[row] rounded to fp16, plane 1 the rounded remainder (23 significant bits kept)
+template <class G>
+static void pack_block_f16x2(unsigned short* blk, int rb, int c, int rows, int K, G get, const int* sh) {
+    for (int j = 0; j < 64; ++j)
+        for (int e = 0; e < 8; ++e) {
+            int row = PG_ROWS * rb + (j & 31);
+            int k = PG_KC * c + 8 * (j >> 5) + e;
+            const double v = (row < rows && k < K) ? std::ldexp((double)get(row, k), sh[j & 31]) : 0.0;
+            double r0;
+            blk[j * 8 + e] = f16_rne(v, &r0);
+            blk[(64 + j) * 8 + e] = f16_rne(v - r0, nullptr);
+        }
+}
+
 // Stream of one (order, parity): for every row block the chunks from its first non-negligible one on.  Towards the
 // poles Pbar_l^m falls off like sin^m(theta) (and faster below the turning latitude sin(theta) = m / l): the leading
 // chunks of a row block whose entries are all at most `thr` in magnitude are left out -- `skip[rb]` of them, the kernel
 // starts that row block's K loop there.  With thr = 2^-64 of the largest entry of the order the omitted terms are 2^-40
 // of one fp32 rounding of the result.
+// PG_FORMAT_F16X2: rinv receives, per row block, the 32 factors 2^-sh that undo the row scales.
 template <class G>
-static void pack_stream(std::vector<float>& out, std::vector<int>& skip, int rows, int K, int format, double thr, G get) {
+static void pack_stream(std::vector<float>& out, std::vector<int>& skip, std::vector<float>& rinv, int rows, int K, int format, double thr, G get) {
     const int nrb = (rows + PG_ROWS - 1) / PG_ROWS, nc = (K + PG_KC - 1) / PG_KC;
     const size_t bf = (size_t)pg_block_floats(format);
     for (int rb = 0; rb < nrb; ++rb) {
@@ -252,11 +285,26 @@ static void pack_stream(std::vector<float>& out, std::vector<int>& skip, int row
             if (!negligible) break;
         }
         skip.push_back(c0);
+        int sh[PG_ROWS];
+        if (format == PG_FORMAT_F16X2) {
+            // the largest entry of a row lands in [2^14, 2^15)
+            for (int r = 0; r < PG_ROWS; ++r) {
+                const int row = PG_ROWS * rb + r;
+                double mx = 0.0;
+                if (row < rows)
+                    for (int k = 0; k < K; ++k) mx = std::max(mx, std::fabs((double)get(row, k)));
+                int e = 0;
+                if (mx > 0.0) (void)std::frexp(mx, &e);           // mx in [2^(e-1), 2^e)
+                sh[r] = mx > 0.0 ? 15 - e : 0;
+                rinv.push_back((float)std::ldexp(1.0, -sh[r]));
+            }
+        }
         const size_t at = out.size();
         out.resize(at + (size_t)(nc - c0) * bf, 0.0f);
         for (int c = c0; c < nc; ++c) {
             float* blk = out.data() + at + (size_t)(c - c0) * bf;
-            if (format == PG_FORMAT_BF16) pack_block_bf16(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get);
+            if (format == PG_FORMAT_F16X2) pack_block_f16x2(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get, sh);
+            else if (format == PG_FORMAT_BF16) pack_block_bf16(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get);
             else if (format == PG_FORMAT_SPLIT) pack_block_split(reinterpret_cast<unsigned short*>(blk), rb, c, rows, K, get);
             else pack_block(blk, rb, c, rows, K, get);
         }
@@ -264,19 +312,23 @@ static void pack_stream(std::vector<float>& out, std::vector<int>& skip, int row
 }
 
 void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double* order_scale, bool analysis, int format,
-                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb) {
+                        std::vector<float>& packed, std::vector<int64_t>& aoff, std::vector<double>* chunks_per_rb, std::vector<float>* rinv) {
     const int mmax = g.mmax, lmax = g.lmax, nlat = g.nlat;
     const int K2 = (nlat + 1) / 2;
     auto nl_p = [&](int m, int p) { return (lmax - m - p > 0) ? (lmax - m - p + 1) / 2 : 0; };
     // per (order, parity): the packed blocks and the number of skipped leading chunks of every row block
     std::vector<std::vector<float>> part((size_t)2 * mmax);
     std::vector<std::vector<int>> skip((size_t)2 * mmax);
+    std::vector<std::vector<float>> rpart((size_t)2 * mmax);          // row factors of the two-part fp16 format, per row-block entry
     parallel_for(mmax, [&](int m) {
         int nl = lmax - m;
         if (nl <= 0) {
             // no degrees: the synthesis still has its row blocks (they produce zeros), each with an empty K loop
             if (!analysis)
-                for (int p = 0; p < 2; ++p) skip[2 * m + p].assign((size_t)(K2 + PG_ROWS - 1) / PG_ROWS, 0);
+                for (int p = 0; p < 2; ++p) {
+                    skip[2 * m + p].assign((size_t)(K2 + PG_ROWS - 1) / PG_ROWS, 0);
+                    if (format == PG_FORMAT_F16X2) rpart[2 * m + p].assign(skip[2 * m + p].size() * PG_ROWS, 1.0f);
+                }
             return;
         }
         std::vector<double> rows((size_t)nl * nlat);
@@ -294,8 +346,8 @@ void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double*
             const int kpad = nl_p(m, 0);
             auto wa = [=](int row, int k) { return r[(size_t)(p + 2 * row) * nlat + k] * lw(k); };
             auto ws = [=](int row, int k) { return k < np ? r[(size_t)(p + 2 * k) * nlat + row] * lw(row) : 0.0; };
-            if (analysis) pack_stream(part[2 * m + p], skip[2 * m + p], np, K2, format, thr, wa);
-            else pack_stream(part[2 * m + p], skip[2 * m + p], K2, kpad, format, thr, ws);
+            if (analysis) pack_stream(part[2 * m + p], skip[2 * m + p], rpart[2 * m + p], np, K2, format, thr, wa);
+            else pack_stream(part[2 * m + p], skip[2 * m + p], rpart[2 * m + p], K2, kpad, format, thr, ws);
         }
     });
     // index: aoff[2 m + p] = position (in aoff) of the first row-block entry of that stream; an entry is
@@ -309,6 +361,11 @@ void pack_legendre_fold(const LegendreGen& g, const double* lat_w, const double*
     aoff.assign((size_t)2 * mmax + nent, 0);
     packed.resize(nfl);
     if (chunks_per_rb) chunks_per_rb->assign(mmax, 0.0);
+    if (rinv) {
+        // one group of 32 factors per row-block entry, in the order of the entries
+        rinv->clear();
+        for (size_t b = 0; b < rpart.size(); ++b) rinv->insert(rinv->end(), rpart[b].begin(), rpart[b].end());
+    }
     size_t ent = (size_t)2 * mmax, blk = 0, fl = 0;
     for (int m = 0; m < mmax; ++m) {
         double kept = 0.0;

@@ -70,7 +70,7 @@ class _Plan:
             check(
                 lib.sfno_sht_plan_create(
                     mod.nlat, mod.nlon, mod.lmax, mod.mmax, _lib.GRID[mod.grid], _lib.NORM[mod.norm], int(mod.csphase), directions,
-                    {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16, "fp32_mfma": _lib.COMPUTE_FP32_MFMA}[mod.compute], ctypes.byref(self.handle),
+                    {"fp32": _lib.COMPUTE_FP32, "bf16": _lib.COMPUTE_BF16, "fp32_mfma": _lib.COMPUTE_FP32_MFMA, "fp32_bf16x3": _lib.COMPUTE_FP32_BF16X3}[mod.compute], ctypes.byref(self.handle),
                 ),
                 "sfno_sht_plan_create",
             )
@@ -100,8 +100,8 @@ class _SHTBase(nn.Module):
         #   bf16 matrix pipe with every operand cut exactly into three bf16 numbers;
         # "fp32_mfma": the same on the fp32 matrix instruction;
         # "bf16": bf16 tables and inputs, fp32 accumulation.
-        if compute not in ("fp32", "bf16", "fp32_mfma"):
-            raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32', 'fp32_mfma' or 'bf16'")
+        if compute not in ("fp32", "bf16", "fp32_mfma", "fp32_bf16x3"):
+            raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32', 'fp32_mfma', 'fp32_bf16x3' or 'bf16'")
         self.compute = compute
         self.nlat = nlat
         self.nlon = nlon

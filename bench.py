@@ -9,7 +9,12 @@ through the reference-layout module interface (RealSHT.forward then
 InverseRealSHT.forward).  One step = one such pair with the input already resident in
 HBM.  Prints ONE JSON line; `roofline` describes the dominant kernel (the Legendre
 contraction) from HIP-event timings taken in this run, `cpu_baseline` is the PyTorch-CPU
-restatement of the reference op sequence timed on this host on a channel sample.
+restatement of the reference op sequence timed on this host on the whole workload
+(--quick: on a channel sample).  The default run appends the other configurations of the
+metric as extra keys, each with its own roofline and CPU baseline: the SFNO-8L forward
+(configs[3], with every kernel class timed at its in-model shape), one spectral block
+(configs[2], fp32 and bf16), the batch-4 rollout (configs[4]) and the Legendre stage on the
+fp32 matrix instruction.
 """
 import argparse
 import ctypes
@@ -24,7 +29,7 @@ for p in (ROOT, os.path.join(ROOT, "modulus-makani_amd")):
         sys.path.insert(0, p)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
-PEAK_BF16_MFMA_TFLOPS = 2500.0
+PEAK_BF16_MFMA_TFLOPS = 2500.0       # dense bf16 and fp16
 PEAK_HBM_GBS = 8000.0
 
 
@@ -35,9 +40,12 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
-    ap.add_argument("--compute", default="fp32", choices=["fp32", "bf16", "fp32_mfma"],
-                    help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision; fp32 operands cut into three bf16 planes on the bf16 "
-                         "matrix pipe), fp32_mfma (transform pair only: the same on the fp32 matrix instruction) or bf16 MFMA inputs with fp32 accumulation")
+    ap.add_argument("--compute", default="fp32", choices=["fp32", "fp32_bf16x3", "bf16", "fp32_mfma"],
+                    help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision: operands scaled and cut into two fp16 parts, "
+                         "three products on the fp16 matrix pipe), fp32_bf16x3 (three exact bf16 parts, six products), fp32_mfma (transform pair only: "
+                         "the fp32 matrix instruction) or bf16 MFMA inputs with fp32 accumulation")
+    ap.add_argument("--no-extras", action="store_true", help="skip the spectral-block, rollout and fp32-MFMA figures appended to the default run")
+    ap.add_argument("--quick", action="store_true", help="CPU baselines on a channel sample (scaled) instead of the whole workload")
     ap.add_argument("--rollout-steps", type=int, default=12, help="autoregressive steps timed by --workload rollout")
     ap.add_argument("--rollout-warmup", type=int, default=2)
     ap.add_argument("--backward", action="store_true", help="--workload spectral_block: time forward + backward (input and weight gradients)")
@@ -124,15 +132,23 @@ def read_traffic(key, note=None):
     return entry.get("bytes")
 
 
-def cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, channels, sample):
-    """Times the reference op sequence (dense fp32 tables, torch.fft + torch.einsum) on the host cores."""
+def cpu_threads():
+    import torch
+
+    torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 1) <= 64 else 64)
+    return torch.get_num_threads()
+
+
+def cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, channels, sample=None):
+    """Times the reference op sequence (dense fp32 tables, torch.fft + torch.einsum) on the host cores: the whole workload
+    (all channels), or -- sample = n -- n channels scaled by n / channels."""
     import torch
     from oracle.torch_ref import TorchRefSHT
 
-    torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 1) <= 64 else 64)
+    cores = cpu_threads()
     ref = TorchRefSHT(nlat, nlon, lmax, mmax, grid)
-    g = torch.Generator().manual_seed(7)
-    x = torch.randn(1, sample, nlat, nlon, generator=g)
+    n = channels if not sample else min(sample, channels)
+    x = torch.randn(1, n, nlat, nlon, generator=torch.Generator().manual_seed(7))
     times = []
     for it in range(4):
         t0 = time.perf_counter()
@@ -140,17 +156,39 @@ def cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, channels, sample):
         dt = time.perf_counter() - t0
         if it:
             times.append(dt)
-    t = min(times)
     assert y.shape == x.shape
-    # the pair is linear in the number of channels: scale the sample to the full workload
+    t = min(times)
+    times.sort()
+    what = (f"the whole workload: {channels} channels" if n == channels else
+            f"{n} of {channels} channels, scaled by {n}/{channels} (the pair is linear in the number of channels)")
     return {
-        "value": (1.0 / t) * (sample / channels),
+        "value": (1.0 / t) * (n / channels),
         "unit": "pairs/s",
-        "cores": torch.get_num_threads(),
+        "cores": cores,
         "kind": "port",
-        "sample": f"{sample} of {channels} channels, full {nlat}x{nlon} grid, all orders, dense fp32 tables; best of 3 after 1 warm-up "
-                  f"({t:.3f} s per sample pair), scaled by {sample}/{channels}",
+        "sample": f"{what}, full {nlat}x{nlon} grid, all orders, dense fp32 tables; best of 3 after 1 warm-up "
+                  f"({t:.3f} s, median {times[1]:.3f} s)",
     }
+
+
+def cpu_baseline_spectral_block(nlat, nlon, L, M, grid, C, weight, sample=None):
+    """configs[2] on the host cores: rfft -> two einsums -> the dhconv einsum (contractions.py:134) -> two einsums -> irfft."""
+    import torch
+    from oracle.torch_ref import TorchRefSHT
+
+    cores = cpu_threads()
+    ref = TorchRefSHT(nlat, nlon, L, M, grid)
+    w = weight.detach().cpu()
+    x = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(2))
+    times = []
+    for it in range(3):
+        t0 = time.perf_counter()
+        y = ref.inverse(torch.einsum("bixy,iox->boxy", ref.forward(x), w))
+        if it:
+            times.append(time.perf_counter() - t0)
+    assert y.shape == x.shape
+    return {"value": 1.0 / min(times), "unit": "blocks/s", "cores": cores, "kind": "port",
+            "sample": f"the whole block ({C} channels, {nlat}x{nlon}), best of 2 after 1 warm-up ({min(times):.3f} s)"}
 
 
 def bench_sht_pair(args):
@@ -216,29 +254,35 @@ def bench_sht_pair(args):
     hbm_gbs = leg_bytes / (stage_ms[dom] * 1e-3) / 1e9
     mfma_view = {"achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                  "algorithmic_flops_per_launch": leg_flops}
+    kname = f"{'legendre_f16_kernel' if args.compute == 'fp32' else 'legendre_fold_kernel'} ({dom})"
     if args.compute == "fp32_mfma":
         # contraction on the fp32 matrix instruction: 45 flop per byte, above the fp32 ridge (19.7)
-        roofline = {"kernel": f"legendre_fold_kernel ({dom})", "bound": "mfma", **mfma_view, "traffic": None,
+        roofline = {"kernel": kname, "bound": "mfma", **mfma_view, "traffic": None,
                     "avg_launch_ms": stage_ms[dom],
                     "note": "algorithmic (triangular) fp32 flops over the kernel's time; the kernel executes half of those MACs (equator fold)"}
     else:
-        # contraction on the bf16 matrix pipe (fp32 operands cut into three bf16 planes, or bf16 operands): 45 flop per byte is
-        # far below that pipe's ridge (312), so HBM is the roofline that bounds the kernel
+        # contraction on the fp16 / bf16 matrix pipe (fp32 operands cut into two fp16 or three bf16 parts, or bf16 operands): 45 flop per
+        # byte is far below that pipe's ridge (312), so HBM is the roofline that bounds the kernel
         tnote = []
-        # what the matrix pipe executes: half the algorithmic MACs (equator fold), each as six bf16 products (one in bf16 mode)
-        executed = leg_flops / 2 * (6 if args.compute == "fp32" else 1)
-        roofline = {"kernel": f"legendre_fold_kernel ({dom})", "bound": "hbm", "achieved": hbm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+        # what the matrix pipe executes: half the algorithmic MACs (equator fold), each as three fp16 / six bf16 products (one in bf16 mode)
+        products = {"fp32": 3, "fp32_bf16x3": 6, "bf16": 1}[args.compute]
+        executed = leg_flops / 2 * products
+        how = {"fp32": " and forms every fp32 product from three fp16 MFMA partial products of operands scaled by powers of two and cut into two fp16 "
+                       "parts (4-byte table entries)",
+               "fp32_bf16x3": " and forms every fp32 product from six bf16 MFMA partial products of exactly split operands (6-byte table entries)",
+               "bf16": ""}[args.compute]
+        roofline = {"kernel": kname, "bound": "hbm", "achieved": hbm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": hbm_gbs / PEAK_HBM_GBS, "traffic": read_traffic(dom, tnote) if args.compute == "fp32" else None,
                     "algorithmic_bytes_per_launch": leg_bytes,
                     "avg_launch_ms": stage_ms[dom], "against_fp32_mfma_peak": mfma_view,
-                    "executed_on_bf16_pipe": {"flops_per_launch": executed, "achieved_TFLOPs": executed / (stage_ms[dom] * 1e-3) / 1e12,
-                                              "peak_TFLOPs": PEAK_BF16_MFMA_TFLOPS, "frac": executed / (stage_ms[dom] * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS},
+                    "executed_on_matrix_pipe": {"products_per_mac": products, "flops_per_launch": executed,
+                                                "achieved_TFLOPs": executed / (stage_ms[dom] * 1e-3) / 1e12,
+                                                "peak_TFLOPs": PEAK_BF16_MFMA_TFLOPS, "frac": executed / (stage_ms[dom] * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS},
                     "traffic_note": tnote[0] if tnote else None,
                     "note": ("algorithmic bytes = Fourier panel + triangular table at the reference's element size + triangular coefficients, "
-                             "each moved once; the kernel folds the equator (half the MACs and table entries)"
-                             + (" and forms every fp32 product from six bf16 MFMA partial products of exactly split operands (6-byte table "
-                                "entries), which takes the contraction off the fp32 matrix roofline: against that peak the same launch reads "
-                                f"{achieved:.0f} of {PEAK_FP32_MFMA_TFLOPS} TFLOP/s" if args.compute == "fp32" else ""))}
+                             "each moved once; the kernel folds the equator (half the MACs and table entries)" + how
+                             + (f", which takes the contraction off the fp32 matrix roofline: against that peak the same launch reads "
+                                f"{achieved:.0f} of {PEAK_FP32_MFMA_TFLOPS} TFLOP/s" if products > 1 else ""))}
     fft_bytes = rows * nlat * nlon * 4 + rows * nlat * mmax * 8
     result = {
         "metric": "SHT fwd+inv/s @721x1440",
@@ -253,6 +297,7 @@ def bench_sht_pair(args):
         "vs_baseline": None,
         "dtype": "f32" if args.compute != "bf16" else "bf16 MFMA inputs, f32 accumulate (FFT f32)",
         "data": "synthetic",
+        "compute": args.compute,
         "config": {
             "workload": "configs[1]: RealSHT + InverseRealSHT, equiangular 721x1440, lmax=mmax=721, batch 1, 73 channels, "
                         "band-limited Gaussian random fields (l^-2 power, unit variance)",
@@ -271,7 +316,7 @@ def bench_sht_pair(args):
     }
     if not args.no_cpu_baseline:
         del xm, spec, coeffs, out
-        result["cpu_baseline"] = cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, C, args.cpu_sample_channels)
+        result["cpu_baseline"] = cpu_baseline_sht_pair(nlat, nlon, lmax, mmax, grid, C, args.cpu_sample_channels if args.quick else None)
     return result
 
 
@@ -348,9 +393,9 @@ def bench_fft2_pair(args):
     if not args.no_cpu_baseline:
         from oracle.torch_ref import TorchRefFFT2
 
-        torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 1) <= 64 else 64)
+        cpu_threads()
         ref = TorchRefFFT2(nlat, nlon)
-        xs = x[:, : 2 * args.cpu_sample_channels].cpu()
+        xs = (x[:, : 2 * args.cpu_sample_channels] if args.quick else x).cpu()
         times = []
         for it in range(4):
             t0 = time.perf_counter()
@@ -413,7 +458,7 @@ def bench_spectral_block(args):
             "unit": "blocks/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "f32" if args.compute == "fp32" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic",
+            "dtype": "f32" if args.compute != "bf16" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic",
             "config": {"workload": "configs[2] with its backward pass: SHT -> dhconv -> inverse SHT, gradients of the input and of the weight"},
             "useful_TFLOPs_per_step": flops / 1e12,
             "achieved_TFLOPs": flops / (dt / args.steps) / 1e12,
@@ -428,17 +473,56 @@ def bench_spectral_block(args):
         torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert torch.isfinite(y).all()
-    return {
+    # the five kernels of the block, each timed on its own through the C ABI on the block's own plans and weight
+    from makani_amd._lib import lib, check
+    from makani_amd.contractions import dhconv_spectral
+
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
+    xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
+    out = torch.empty_like(x)
+    iters = max(5, args.steps)
+    with torch.no_grad():
+        stages = {
+            "rfft": event_time_ms(lambda: check(lib.sfno_rfft(pf, P(x), 0, P(xm), C, sp), "rfft"), iters, stream),
+            "legendre_analysis": event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream),
+            "dhconv": event_time_ms(lambda: dhconv_spectral(spec, conv.weight, 1, M, compute=args.compute), iters, stream),
+            "legendre_synthesis": event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream),
+            "irfft": event_time_ms(lambda: check(lib.sfno_irfft(pi, P(xm), P(out), 0, C, sp), "irfft"), iters, stream),
+        }
+    wbytes = 4 if args.compute == "bf16" else 8
+    work = {   # algorithmic bytes per launch
+        "rfft": C * nlat * nlon * 4 + C * nlat * M * 8, "irfft": C * nlat * nlon * 4 + C * nlat * M * 8,
+        "legendre_analysis": C * nlat * M * 8 + triangular_count(L, M) * nlat * (2 if args.compute == "bf16" else 4) + C * Tp * 8,
+        "dhconv": C * C * L * wbytes + 2 * C * Tp * 8,
+    }
+    work["legendre_synthesis"] = work["legendre_analysis"]
+    dom = max(stages, key=lambda k: stages[k])
+    gbs = work[dom] / (stages[dom] * 1e-3) / 1e9
+    res = {
         "metric": "spectral block fwd/s @241x480x384",
         "value": args.steps / dt,
         "unit": "blocks/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.compute == "fp32" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic",
+        "dtype": "f32" if args.compute != "bf16" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic", "compute": args.compute,
         "config": {"workload": "configs[2]: SHT -> dhconv -> inverse SHT, legendre-gauss 241x480, lmax=mmax=241, batch 1, 384 channels"},
         "useful_TFLOPs_per_step": (dh_flops + 2 * leg_flops) / 1e12,
         "achieved_TFLOPs": (dh_flops + 2 * leg_flops) / (dt / args.steps) / 1e12,
+        "stages_ms": stages,
+        # at batch 1 every kernel of the block is below the ridge of the matrix pipe it runs on: HBM bounds it
+        "roofline": {"kernel": dom, "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                     "traffic": read_traffic("block_" + dom) if args.compute == "fp32" else None, "algorithmic_bytes_per_launch": work[dom],
+                     "avg_launch_ms": stages[dom],
+                     "per_stage_frac": {k: work[k] / (stages[k] * 1e-3) / 1e9 / PEAK_HBM_GBS for k in stages}},
     }
+    if not args.no_cpu_baseline:
+        del xm, spec, out
+        res["cpu_baseline"] = cpu_baseline_spectral_block(nlat, nlon, L, M, "legendre-gauss", C, conv.weight)
+    return res
 
 
 def build_sfno8l(dev, compute="fp32"):
@@ -517,7 +601,7 @@ def sfno_kernel_classes(dev, net, iters=10):
         T = triangular_count(lmax, mmax)
         Tp = sum(min(l + 1, mmax) for l in range(lmax))
         leg_bytes = C * nlat * mmax * 8 + T * nlat * 4 + C * Tp * 8
-        leg_flops = 4.0 * C * nlat * T / 2 * 6          # executed: equator fold, six bf16 products per fp32 product
+        leg_flops = 4.0 * C * nlat * T / 2 * 3          # executed: equator fold, three fp16 products per fp32 product
         t = event_time_ms(lambda: check(lib.sfno_rfft(pf, P(x), _lib.DTYPE_BF16, P(xm), C, sp), "rfft"), iters, stream)
         hbm(f"rfft {tag} bf16 in", n_r, t, fft_bytes)
         t = event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream)
@@ -530,7 +614,7 @@ def sfno_kernel_classes(dev, net, iters=10):
             from makani_amd.contractions import dhconv_spectral
             w = net.blocks[1].filter.filter.weight
             t = event_time_ms(lambda: dhconv_spectral(spec, w, 1, mmax), iters, stream)
-            mfma("dhconv 384x384x240", nl, t, 8.0 * C * C * Tp * 6 / 4 * 2, C * C * lmax * 8 + 2 * C * Tp * 8)
+            mfma("dhconv 384x384x240", nl, t, 8.0 * C * C * Tp * 3, C * C * lmax * 8 + 2 * C * Tp * 8)      # executed: three fp16 products per real product
         del x, xm, spec
     # 1x1 convolutions of the pointwise tail: (name, module weight, bias, act, addend?, resolution, calls)
     hw_big, hw_small = net.inp_shape, (net.h, net.w)
@@ -604,7 +688,7 @@ def bench_sfno8l(args):
     return {
         "metric": "SFNO-L8 fwd ms/sample", "value": med, "unit": "ms/sample", "n_gpus": 1, "steps": max(args.steps, 5), "warmup": args.warmup,
         "ms_per_step": med, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 pointwise / f32 spectral" if args.compute == "fp32" else "bf16 pointwise / bf16-MFMA spectral contractions",
+        "dtype": "bf16 pointwise / f32 spectral" if args.compute != "bf16" else "bf16 pointwise / bf16-MFMA spectral contractions",
         "data": "synthetic",
         "config": {"workload": "configs[3]: SFNO-linear 8 layers, embed 384, scale factor 3 (721x1440 -> 240x480), 73 channels, batch 1, "
                                "bf16 autocast forward, random-init weights, N(0,1) inputs"},
@@ -644,7 +728,42 @@ def bench_rollout(args):
         "config": {"workload": "configs[4]: SFNO-8L, batch 4, 12-step autoregressive rollout, bf16 autocast"},
         "ms_per_sample_step": dt / nsteps / 4 * 1e3, "finite": finite,
         "hbm_traffic_bytes_per_step": traffic, "hbm_traffic_bytes_total": traffic * nsteps if traffic else None,
+        # the whole step as one HBM stream: measured bytes of all its kernels (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/) over its time
+        "roofline": ({"kernel": "all kernels of one rollout step (batch 4)", "bound": "hbm", "achieved": traffic / (dt / nsteps) / 1e9, "peak": PEAK_HBM_GBS,
+                      "unit": "GB/s", "frac": traffic / (dt / nsteps) / 1e9 / PEAK_HBM_GBS, "traffic": traffic,
+                      "note": "measured traffic, not algorithmic bytes: the per-kernel algorithmic figures are in sfno_l8_fwd_ms_per_sample.kernel_classes"}
+                     if traffic else None),
+        "cpu_baseline": {"value": None, "unit": "ms/step", "cores": os.cpu_count(), "kind": "port",
+                         "sample": "skipped: budget (one sample of the 8-layer network is 4.5 TFLOP of fp32 convolutions on the host; the transform "
+                                   "pair and the spectral block carry the CPU comparison)"},
     }
+
+
+def legendre_fp32_mfma_figure(iters=10):
+    """The Legendre stage of configs[1] on the fp32 matrix instruction (compute="fp32_mfma"): time per direction and algorithmic
+    (triangular) flops over it against the fp32 MFMA peak."""
+    import torch
+    import makani_amd as ma
+    from makani_amd._lib import lib, check
+
+    dev = torch.device("cuda:0")
+    nlat, nlon, lmax, mmax, C = 721, 1440, 721, 721, 73
+    sht = ma.RealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid="equiangular", compute="fp32_mfma")
+    isht = ma.InverseRealSHT(nlat, nlon, lmax=lmax, mmax=mmax, grid="equiangular", compute="fp32_mfma")
+    x = make_fields(isht, C, dev)
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
+    xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
+    check(lib.sfno_rfft(pf, P(x), 0, P(xm), C, sp), "rfft")
+    ana = event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream)
+    syn = event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream)
+    flops = 4.0 * C * nlat * triangular_count(lmax, mmax)
+    fig = lambda ms: {"ms": ms, "TFLOPs": flops / ms / 1e9, "frac": flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+    return {"analysis": fig(ana), "synthesis": fig(syn), "peak_TFLOPs": PEAK_FP32_MFMA_TFLOPS, "algorithmic_flops_per_launch": flops,
+            "note": "v_mfma_f32_32x32x2_f32 on fp32 tables; algorithmic (triangular) flops, of which the kernel executes half (equator fold)"}
 
 
 def main():
@@ -674,6 +793,30 @@ def main():
                                                 "config": "configs[3]: SFNO-linear 8 layers, embed 384, 721x1440, 73 channels, bf16 autocast",
                                                 "kernel_classes_ms_sum": sum(c["calls"] * c["ms"] for c in classes.values()),
                                                 "kernel_classes": classes}
+            del net, classes
+        if not args.no_extras and args.compute == "fp32":
+            import copy
+            import gc
+
+            def sub(workload, compute, steps, warmup):
+                a = copy.copy(args)
+                a.workload, a.compute, a.steps, a.warmup, a.backward = workload, compute, steps, warmup, False
+                gc.collect()
+                torch.cuda.empty_cache()
+                return a
+
+            keep = ("value", "unit", "ms_per_step", "dtype", "compute", "config", "stages_ms", "roofline", "cpu_baseline", "achieved_TFLOPs",
+                    "ms_per_sample_step", "finite", "hbm_traffic_bytes_per_step", "hbm_traffic_bytes_total", "steps", "warmup")
+            pick = lambda r: {k: r[k] for k in keep if k in r}
+            # configs[2] in both variants, configs[4], and the Legendre stage on the fp32 matrix instruction
+            res["spectral_block"] = {"fp32": pick(bench_spectral_block(sub("spectral_block", "fp32", 20, 5)))}
+            a = sub("spectral_block", "bf16", 20, 5)
+            a.no_cpu_baseline = True          # same host computation as the fp32 variant
+            res["spectral_block"]["bf16"] = pick(bench_spectral_block(a))
+            res["rollout"] = pick(bench_rollout(sub("rollout", "fp32", 12, 2)))
+            gc.collect()
+            torch.cuda.empty_cache()
+            res["legendre_fp32_mfma"] = legendre_fp32_mfma_figure()
     elif args.workload == "fft2_pair":
         res = bench_fft2_pair(args)
     elif args.workload == "spectral_block":

@@ -259,7 +259,7 @@ def _contract_dense(x, weight, separable=False, operator_type="diagonal", comple
     The separable variants are not provided: the reference's einsums for them ("bixy,ixy->boxy", "bixy,ix->boxy",
     contractions.py:139-154) name an output index that no input carries, so they cannot be evaluated there either."""
     if operator_type not in ("diagonal", "dhconv"):
-        raise ValueError(f"Unkonw operator type {operator_type}")
+        raise ValueError(f"unknown operator type {operator_type!r}, expected 'diagonal' or 'dhconv'")
     if separable or not complex:
         raise NotImplementedError("only the non-separable complex operators run on the HIP path")
     if operator_type == "diagonal":

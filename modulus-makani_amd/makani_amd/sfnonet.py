@@ -65,8 +65,15 @@ def _run_chain(steps, x, addend=None, add_scale=None, add_shift=None):
     return x
 
 
+def _stamp(*tensors):
+    """Identity of the current values of some parameters, for the caches of tensors derived from them: storage address and
+    version counter (inference tensors have none: they cannot be updated in place)."""
+    return tuple((t.data_ptr(), -1 if t.is_inference() else t._version) for t in tensors)
+
+
 def fused_pointwise_active(x):
-    """The fused kernels serve inference on bf16 activations: bf16 input or bf16 autocast, and no autograd graph."""
+    """The fused kernels serve inference on bf16 activations: bf16 input or bf16 autocast, and no autograd graph (the callers
+    also require ``eval()`` mode: a module in training mode always runs the PyTorch modules)."""
     if torch.is_grad_enabled() or not x.is_cuda or x.dim() != 4:
         return False
     bf16 = x.dtype == torch.bfloat16 or (torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16)
@@ -214,12 +221,12 @@ class FourierNeuralOperatorBlock(nn.Module):
 
     def forward(self, x, defer_skip=False):
         # on the fused inference path the inverse transform hands over the moments norm0 needs together with its output
-        want_stats = getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and self._fusable()
+        want_stats = getattr(self, "fused_pointwise", True) and not self.training and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and self._fusable()
         if want_stats:
             x, residual, lat_stats = self.filter(x, lat_stats=True)
         else:
             (x, residual), lat_stats = self.filter(x), None
-        if getattr(self, "fused_pointwise", True) and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 \
+        if getattr(self, "fused_pointwise", True) and not self.training and fused_pointwise_active(x) and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 \
                 and residual.shape[2:] == x.shape[2:] and self._fusable():
             return self._forward_fused(x.contiguous(), residual.contiguous(), lat_stats, defer_skip=defer_skip)
         # (defer_skip is honoured on the fused path only; here the block's output comes back whole)
@@ -373,12 +380,16 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         conv = blk.filter.filter
         if enc is None or len(enc) < 2 or enc[-1][1] is not None or enc[-1][0].bias is not None:
             return None
+        # the fold moves the first block's transforms, channel mix and skip convolution from the encoder's output channels to
+        # its hidden channels: worth it only if those are not more
+        if enc[-1][0].in_channels > enc[-1][0].out_channels:
+            return None
         if not (isinstance(blk, FourierNeuralOperatorBlock) and blk._fusable() and getattr(blk, "fused_pointwise", True)):
             return None
         if not (conv._fused and conv.scale_residual and not hasattr(conv, "bias") and conv.in_channels == enc[-1][0].out_channels):
             return None
         w2, w0, ws = enc[-1][0].weight, conv.weight, blk.outer_skip.weight
-        stamp = tuple((t.data_ptr(), t._version) for t in (w2, w0, ws))
+        stamp = _stamp(w2, w0, ws)
         cached = getattr(self, "_fold_cache", None)
         if cached is None or cached[0] != stamp:
             # (ordinary tensors, also when called under inference_mode: the packed-operand caches read version counters)
@@ -430,7 +441,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
     def _tail_weight(self, conv):
         """[W_last | W_res] of the decoder's last convolution and residual_transform, cached until one of them changes."""
         wl, wr = conv.weight, self.residual_transform.weight
-        stamp = tuple((t.data_ptr(), t._version) for t in (wl, wr))
+        stamp = _stamp(wl, wr)
         cached = getattr(self, "_tail_cache", None)
         if cached is None or cached[0] != stamp:
             with torch.inference_mode(False), torch.no_grad():
@@ -451,7 +462,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         B, C = m.shape[:2]
         with torch.inference_mode(False), torch.no_grad():
             cached = getattr(self, "_merge_cache", None)
-            stamp = tuple((t.data_ptr(), t._version) for t in (conv_d.weight, blk.outer_skip.weight))
+            stamp = _stamp(conv_d.weight, blk.outer_skip.weight)
             if cached is None or cached[0] != stamp:
                 wd = conv_d.weight.detach().reshape(conv_d.weight.shape[0], -1).to(torch.bfloat16).float()
                 ws = blk.outer_skip.weight.detach().reshape(C, -1).to(torch.bfloat16).float()
@@ -517,7 +528,7 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
         return _run_chain(dec, x, residual if self.big_skip else None)
 
     def _fusable(self, x):
-        if not (getattr(self, "fused_pointwise", True) and fused_pointwise_active(x)) or hasattr(self, "pos_embed"):
+        if not (getattr(self, "fused_pointwise", True) and not self.training and fused_pointwise_active(x)) or hasattr(self, "pos_embed"):
             return False
         if not isinstance(self.pos_drop, nn.Identity) or (self.out_shape[0] * self.out_shape[1]) % 8 != 0:
             return False

@@ -14,64 +14,55 @@ from .sht import RealSHT, InverseRealSHT
 class SpectralConv(nn.Module):
     """Spectral convolution on the sphere: SHT -> per-degree complex channel mix -> inverse SHT."""
 
+    # per-mode extent of the weight behind [in_channels, out_channels]: the contract of spectral_convolution.py:89-96
+    _MODE_DIMS = {"diagonal": ("modes_lat_local", "modes_lon_local"), "dhconv": ("modes_lat_local",)}
+
     def __init__(self, forward_transform, inverse_transform, in_channels, out_channels, operator_type="diagonal", separable=False, bias=False, gain=1.0,
                  compute="fp32"):
+        """Attribute names, the shape of ``weight`` and its initial distribution are those of the reference module
+        (spectral_convolution.py:50-122), so that its checkpoints load and its callers find what they read.
+
+        compute: arithmetic of the channel mix -- "fp32" (default, the reference's precision), "fp32_bf16x3" or "bf16"
+        (bf16 matrix inputs, fp32 accumulation)."""
         super().__init__()
-        # compute = "bf16" runs the channel mix on bf16 MFMA (fp32 accumulate); the reference and the default stay fp32
-        self.compute = compute
-        self.forward_transform = forward_transform
-        self.inverse_transform = inverse_transform
-        self.in_channels = in_channels
-        self.out_channels = out_channels
-        self.modes_lat = self.inverse_transform.lmax
-        self.modes_lon = self.inverse_transform.mmax
-        self.scale_residual = (self.forward_transform.nlat != self.inverse_transform.nlat) or (self.forward_transform.nlon != self.inverse_transform.nlon)
-        if hasattr(self.forward_transform, "grid"):
-            self.scale_residual = self.scale_residual or (self.forward_transform.grid != self.inverse_transform.grid)
-        self.operator_type = operator_type
-        self.separable = separable
-        assert self.inverse_transform.lmax == self.modes_lat
-        assert self.inverse_transform.mmax == self.modes_lon
-
-        weight_shape = [in_channels]
-        if not self.separable:
-            weight_shape += [out_channels]
-        self.modes_lat_local = self.modes_lat
-        self.modes_lon_local = self.modes_lon
-        self.nlat_local = self.inverse_transform.nlat
-        self.nlon_local = self.inverse_transform.nlon
-        if self.operator_type == "diagonal":
-            weight_shape += [self.modes_lat_local, self.modes_lon_local]
-        elif self.operator_type == "dhconv":
-            weight_shape += [self.modes_lat_local]
-        else:
-            raise ValueError(f"Unsupported operator type f{self.operator_type}")
-        if self.separable:
+        if operator_type not in self._MODE_DIMS:
+            raise ValueError(f"unsupported operator type {operator_type!r}, expected one of {sorted(self._MODE_DIMS)}")
+        if separable:
             raise NotImplementedError("the HIP path implements the non-separable operators")
+        fwd, inv = forward_transform, inverse_transform
+        self.forward_transform, self.inverse_transform = fwd, inv
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.operator_type, self.separable, self.compute = operator_type, separable, compute
 
-        # same initialisation as the reference (spectral_convolution.py:97-102)
-        scale = math.sqrt(gain / in_channels) * torch.ones(self.modes_lat_local, dtype=torch.complex64)
-        scale[0] *= math.sqrt(2.0)
-        init = scale * torch.randn(*weight_shape, dtype=torch.complex64)
-        self.weight = nn.Parameter(init)
+        # the filter lives on the modes of the inverse transform; one process holds all of them
+        self.modes_lat = self.modes_lat_local = inv.lmax
+        self.modes_lon = self.modes_lon_local = inv.mmax
+        self.nlat_local, self.nlon_local = inv.nlat, inv.nlon
+        # input and output grids differ: the residual then has to pass through the transforms as well (forward)
+        same_grid = (fwd.nlat, fwd.nlon) == (inv.nlat, inv.nlon) and getattr(fwd, "grid", None) == getattr(inv, "grid", None)
+        self.scale_residual = not same_grid
 
+        # weight ~ sqrt(gain / in_channels) * CN(0, 1) per mode, the degree-0 row larger by sqrt(2)
+        shape = (in_channels, out_channels) + tuple(getattr(self, d) for d in self._MODE_DIMS[operator_type])
+        std = torch.full((self.modes_lat_local,), math.sqrt(gain / in_channels), dtype=torch.complex64)
+        std[0] *= math.sqrt(2.0)
+        # (broadcast along the last axis of the weight: the degree axis for dhconv)
+        self.weight = nn.Parameter(std * torch.randn(*shape, dtype=torch.complex64))
         self._contract = get_contract_fun(self.weight, implementation="factorized", separable=separable, complex=True, operator_type=operator_type)
 
-        if bias == "constant":
-            self.bias = nn.Parameter(torch.zeros(1, self.out_channels, 1, 1))
-        elif bias == "position":
-            self.bias = nn.Parameter(torch.zeros(1, self.out_channels, self.nlat_local, self.nlon_local))
+        bias_shape = {"constant": (1, out_channels, 1, 1), "position": (1, out_channels, self.nlat_local, self.nlon_local)}.get(bias)
+        if bias_shape is not None:
+            self.bias = nn.Parameter(torch.zeros(bias_shape))
 
+        # forward transform -> dhconv -> inverse transform without leaving the order-major spectral layout
         self._fused = (
             operator_type == "dhconv"
-            and isinstance(forward_transform, RealSHT)
-            and isinstance(inverse_transform, InverseRealSHT)
-            and forward_transform.lmax == inverse_transform.lmax
-            and forward_transform.mmax == inverse_transform.mmax
-            and forward_transform._planar == inverse_transform._planar
+            and isinstance(fwd, RealSHT)
+            and isinstance(inv, InverseRealSHT)
+            and (fwd.lmax, fwd.mmax, fwd._planar) == (inv.lmax, inv.mmax, inv._planar)
         )
         # coefficients of a spherical transform vanish for l < m; the planar pair fills the whole rectangle
-        self._triangular = not getattr(forward_transform, "_planar", False)
+        self._triangular = not getattr(fwd, "_planar", False)
 
     def invalidate_packed(self):
         """Drops the packed MFMA operand copies of ``weight``; call after writing the parameter through ``.data``."""

@@ -251,6 +251,63 @@ def test_encoder_fold_matches_layer_by_layer(lib_built):
         assert other._fold_cache is None and torch.isfinite(y.float()).all()
 
 
+def test_fused_path_needs_eval_mode(lib_built):
+    """In training mode the network runs the PyTorch modules even under no_grad and bf16 autocast (a validation pass inside a
+    training loop then follows the training forward's arithmetic); eval() switches the fused kernels on."""
+    case = dict(inp_shape=(48, 96), out_shape=(48, 96), inp_chans=4, out_chans=3, scale_factor=2, embed_dim=32, num_layers=2)
+    net = build(**case).cuda()
+    x = torch.randn(1, 4, 48, 96, generator=torch.Generator().manual_seed(13)).cuda()
+    net.train()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y_train = net(x)
+    assert net._fold_cache is None                      # the fused forward (which folds the encoder) was not taken
+    net.eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y_eval = net(x)
+    assert net._fold_cache is not None
+    assert rel_l2(y_eval.float().cpu().numpy(), y_train.float().cpu().numpy()) < 3e-2
+
+
+def test_network_built_under_inference_mode(lib_built):
+    """A network whose parameters are inference tensors (built and moved to the device under torch.inference_mode()) takes the
+    fused path with the encoder fold and the merged decoder: the caches of derived weights must not ask such tensors for a
+    version counter.  Same output as the same state dict in ordinary tensors."""
+    case = dict(inp_shape=(92, 180), out_shape=(92, 180), inp_chans=5, out_chans=5, scale_factor=3, embed_dim=128, num_layers=3)
+    print(f"case sfno inference-mode parameters {case}", flush=True)
+    with torch.inference_mode():
+        net_inf = build(**case).cuda().eval()
+    assert all(p.is_inference() for p in net_inf.parameters())
+    net = build(**case).cuda().eval()
+    net.load_state_dict({k: v.clone() for k, v in net_inf.state_dict().items()})
+    x = torch.randn(2, 5, 92, 180, generator=torch.Generator().manual_seed(9)).cuda()
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y_inf = net_inf(x)
+        y = net(x)
+    assert net_inf._fold_cache is not None and net_inf._merge_cache is not None and net_inf._tail_cache is not None
+    assert torch.equal(y_inf, y)
+
+
+def test_encoder_fold_not_taken_when_it_widens(lib_built):
+    """encoder_ratio = 2: the encoder's hidden layer is wider than the embedding, so folding its last convolution into block 0
+    would run the transforms on twice the channels; the network then evaluates layer by layer (and agrees with the oracle)."""
+    case = dict(inp_shape=(48, 96), out_shape=(48, 96), inp_chans=4, out_chans=3, scale_factor=2, embed_dim=32, num_layers=2, encoder_ratio=2)
+    print(f"case sfno wide encoder {case}", flush=True)
+    net = build(**case).cuda().eval()
+    x = torch.randn(1, 4, 48, 96, generator=torch.Generator().manual_seed(10))
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = net(x.cuda())
+    assert net._fold_cache is None
+    # (the same network with encoder_ratio = 1 does take the fold: the size is one the fused path accepts)
+    narrow = build(**{**case, "encoder_ratio": 1}).cuda().eval()
+    with torch.inference_mode(), torch.autocast("cuda", dtype=torch.bfloat16):
+        narrow(x.cuda())
+    assert narrow._fold_cache is not None
+    # the bf16 forward is held against the fp32 forward of the same network (itself pinned against the oracle above)
+    with torch.inference_mode():
+        y32 = net(x.cuda())
+    assert rel_l2(y.float().cpu().numpy(), y32.float().cpu().numpy()) < 2e-2
+
+
 def test_decoder_merge_matches_layer_by_layer(lib_built):
     """merge_decoder: the last block's "norm1(mlp) + outer_skip(residual)" and the decoder's first convolution are one convolution
     over the two tensors (both steps are linear), with per-sample weights [W_d diag(scale) | W_d W_skip] and bias W_d shift + b_d.

@@ -280,8 +280,21 @@ constexpr int DM_XBASE = DM_WSTAGES * DM_ABYTES;
 constexpr int DM_LDS = DM_XBASE + DM_XSTAGES * DM_XBYTES;
 static_assert(DM_LDS <= 160 * 1024, "one workgroup per CU");
 
+// M0 carries the LDS destination.  The compiler refuses "m0" in a clobber list (a reserved register), so nothing may
+// keep a value in M0 across this call: the kernels that use it index no register array dynamically and use no
+// readlane/movrel/sendmsg around it.
 __device__ __forceinline__ void dma16(const void* g, unsigned lds_byte_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_addr) : "memory");
+}
+
+// Workgroup barrier of the streaming pipeline: the s_waitcnt in front of it names both counters it depends on (the
+// vector-memory count that leaves later chunks in flight, and lgkmcnt(0) for this wavefront's LDS reads of the chunk
+// that is about to be overwritten), so the barrier itself is the bare instruction and no fence lowering can add a
+// full vmcnt(0) to it.
+__device__ __forceinline__ void dm_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // GELU: exact GELU on the output; ADD: "+ scale * addend + shift"
@@ -370,10 +383,10 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
     bool full = true;
     for (int i = 0; i < (wload ? DM_WSTAGES : DM_XSTAGES); ++i) full = issue() && full;
     if (full)
-        __builtin_amdgcn_s_waitcnt(0x0F7C);        // vmcnt(12): two chunks of weights, three of the four later activation chunks
+        __builtin_amdgcn_s_waitcnt(0x007C);        // vmcnt(12) lgkmcnt(0): two chunks of weights, three of the four later activation chunks
     else
-        __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
-    __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+    dm_barrier();
 
     const unsigned char* abase = lds + (DM_MT * wo) * 1024 + lane * 16;
     const unsigned char* xbase = lds + DM_XBASE + (4 * ko) * DM_XBLK + wp * 256 + 8 * q;
@@ -514,12 +527,12 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
             // read; in flight may stay the loads of one weight chunk (6) or of three activation chunks (12), everything once
             // the stream has run dry.  Then this chunk's stages take the chunk three (five) further on.
             if (!full)
-                __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
+                __builtin_amdgcn_s_waitcnt(0x0070);    // vmcnt(0) lgkmcnt(0)
             else if (wload)
-                __builtin_amdgcn_s_waitcnt(0x0F76);    // vmcnt(6)
+                __builtin_amdgcn_s_waitcnt(0x0076);    // vmcnt(6) lgkmcnt(0)
             else
-                __builtin_amdgcn_s_waitcnt(0x0F7C);    // vmcnt(12)
-            __syncthreads();
+                __builtin_amdgcn_s_waitcnt(0x007C);    // vmcnt(12) lgkmcnt(0)
+            dm_barrier();
             full = issue();
             sw = (sw == DM_WSTAGES - 1) ? 0 : sw + 1;
             sx = (sx == DM_XSTAGES - 1) ? 0 : sx + 1;

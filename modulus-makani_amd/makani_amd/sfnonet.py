@@ -473,16 +473,14 @@ class SphericalFourierNeuralOperatorNet(nn.Module):
                 sc = torch.ones((B, C), dtype=torch.float32, device=m.device)
                 sh = torch.zeros_like(sc)
             sc, sh = sc.clone(), sh.clone()          # ordinary tensors for the arithmetic below
-            outs = []
-            for b in range(B):
-                wcat = torch.cat([wd * sc[b][None, :], wds], dim=1).contiguous()
-                bias = wd @ sh[b]
-                if conv_d.bias is not None:
-                    bias = bias + conv_d.bias.detach().float()
-                outs.append((wcat, bias))
+            # all samples at once: [W_d diag(scale_b) | W_d W_skip] and W_d shift_b (+ bias); only the left half depends on b
+            wcat = torch.cat([wd[None] * sc[:, None, :], wds[None].expand(B, -1, -1)], dim=2).contiguous()
+            bias = sh @ wd.t()
+            if conv_d.bias is not None:
+                bias = bias + conv_d.bias.detach().float()
         y = torch.empty((B, wd.shape[0], m.shape[2], m.shape[3]), dtype=torch.bfloat16, device=m.device)
-        for b, (wcat, bias) in enumerate(outs):
-            pw.conv1x1_cat(m[b:b + 1], r[b:b + 1], wcat, bias, dec[0][1], out=y[b:b + 1])
+        for b in range(B):
+            pw.conv1x1_cat(m[b:b + 1], r[b:b + 1], wcat[b], bias[b], dec[0][1], out=y[b:b + 1])
         return y, dec[1:]
 
     def _forward_fused(self, x):

@@ -48,6 +48,7 @@ def parse():
     ap.add_argument("--quick", action="store_true", help="CPU baselines on a channel sample (scaled) instead of the whole workload")
     ap.add_argument("--rollout-steps", type=int, default=12, help="autoregressive steps timed by --workload rollout")
     ap.add_argument("--rollout-warmup", type=int, default=2)
+    ap.add_argument("--batch", type=int, default=1, help="--workload spectral_block: samples per step (configs[2] is batch 1)")
     ap.add_argument("--backward", action="store_true", help="--workload spectral_block: time forward + backward (input and weight gradients)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--yardstick", action="store_true",
@@ -425,15 +426,17 @@ def bench_spectral_block(args):
     w = torch.complex(torch.randn(C, C, L, generator=g), torch.randn(C, C, L, generator=g)) / (2.0 ** 0.5) * (1.0 / C) ** 0.5
     with torch.no_grad():
         conv.weight.copy_(w.to(dev))
-    x = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(2)).to(dev)
+    B = max(1, args.batch)
+    R = B * C                               # rows of the transforms
+    x = torch.randn(B, C, nlat, nlon, generator=torch.Generator().manual_seed(2)).to(dev)
     Tp = sum(min(l + 1, M) for l in range(L))
-    dh_flops = 8.0 * C * C * Tp
-    leg_flops = 4.0 * C * nlat * triangular_count(L, M)
+    dh_flops = 8.0 * B * C * C * Tp
+    leg_flops = 4.0 * R * nlat * triangular_count(L, M)
     if args.backward:
         # forward + backward (input and weight gradients) through the adjoint kernels: twice the transform work and
         # three times the channel mix of the forward pass
         x.requires_grad_(True)
-        gy = torch.randn(1, C, nlat, nlon, generator=torch.Generator().manual_seed(6)).to(dev)
+        gy = torch.randn(B, C, nlat, nlon, generator=torch.Generator().manual_seed(6)).to(dev)
 
         def step():
             conv.weight.grad = None
@@ -463,6 +466,10 @@ def bench_spectral_block(args):
             "useful_TFLOPs_per_step": flops / 1e12,
             "achieved_TFLOPs": flops / (dt / args.steps) / 1e12,
         }
+    if args.yardstick:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.mul(src, 1.0)            # reads 256 MiB, writes 256 MiB
+        del src, dst
     with torch.no_grad():
         for _ in range(args.warmup):
             conv(x)
@@ -481,23 +488,23 @@ def bench_spectral_block(args):
     sp = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
-    xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
-    spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
+    xm = torch.empty(lib.sfno_fourier_elems(pf, R), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, R), dtype=torch.float32, device=dev)
     out = torch.empty_like(x)
     iters = max(5, args.steps)
     with torch.no_grad():
         stages = {
-            "rfft": event_time_ms(lambda: check(lib.sfno_rfft(pf, P(x), 0, P(xm), C, sp), "rfft"), iters, stream),
-            "legendre_analysis": event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream),
-            "dhconv": event_time_ms(lambda: dhconv_spectral(spec, conv.weight, 1, M, compute=args.compute), iters, stream),
-            "legendre_synthesis": event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream),
-            "irfft": event_time_ms(lambda: check(lib.sfno_irfft(pi, P(xm), P(out), 0, C, sp), "irfft"), iters, stream),
+            "rfft": event_time_ms(lambda: check(lib.sfno_rfft(pf, P(x), 0, P(xm), R, sp), "rfft"), iters, stream),
+            "legendre_analysis": event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), R, sp), "analysis"), iters, stream),
+            "dhconv": event_time_ms(lambda: dhconv_spectral(spec, conv.weight, B, M, compute=args.compute), iters, stream),
+            "legendre_synthesis": event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), R, sp), "synthesis"), iters, stream),
+            "irfft": event_time_ms(lambda: check(lib.sfno_irfft(pi, P(xm), P(out), 0, R, sp), "irfft"), iters, stream),
         }
     wbytes = 4 if args.compute == "bf16" else 8
     work = {   # algorithmic bytes per launch
-        "rfft": C * nlat * nlon * 4 + C * nlat * M * 8, "irfft": C * nlat * nlon * 4 + C * nlat * M * 8,
-        "legendre_analysis": C * nlat * M * 8 + triangular_count(L, M) * nlat * (2 if args.compute == "bf16" else 4) + C * Tp * 8,
-        "dhconv": C * C * L * wbytes + 2 * C * Tp * 8,
+        "rfft": R * nlat * nlon * 4 + R * nlat * M * 8, "irfft": R * nlat * nlon * 4 + R * nlat * M * 8,
+        "legendre_analysis": R * nlat * M * 8 + triangular_count(L, M) * nlat * (2 if args.compute == "bf16" else 4) + R * Tp * 8,
+        "dhconv": C * C * L * wbytes + 2 * R * Tp * 8,
     }
     work["legendre_synthesis"] = work["legendre_analysis"]
     dom = max(stages, key=lambda k: stages[k])
@@ -505,21 +512,23 @@ def bench_spectral_block(args):
     res = {
         "metric": "spectral block fwd/s @241x480x384",
         "value": args.steps / dt,
+        "batch": B,
         "unit": "blocks/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if args.compute != "bf16" else "bf16 MFMA inputs, f32 accumulate (FFT f32)", "data": "synthetic", "compute": args.compute,
-        "config": {"workload": "configs[2]: SHT -> dhconv -> inverse SHT, legendre-gauss 241x480, lmax=mmax=241, batch 1, 384 channels"},
+        "config": {"workload": f"configs[2]: SHT -> dhconv -> inverse SHT, legendre-gauss 241x480, lmax=mmax=241, batch {B}, 384 channels"},
         "useful_TFLOPs_per_step": (dh_flops + 2 * leg_flops) / 1e12,
         "achieved_TFLOPs": (dh_flops + 2 * leg_flops) / (dt / args.steps) / 1e12,
         "stages_ms": stages,
         # at batch 1 every kernel of the block is below the ridge of the matrix pipe it runs on: HBM bounds it
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                     "traffic": read_traffic("block_" + dom) if args.compute == "fp32" else None, "algorithmic_bytes_per_launch": work[dom],
+                     "traffic": read_traffic(("block_" if B == 1 else f"block_b{B}_") + dom) if args.compute == "fp32" else None,
+                     "algorithmic_bytes_per_launch": work[dom],
                      "avg_launch_ms": stages[dom],
                      "per_stage_frac": {k: work[k] / (stages[k] * 1e-3) / 1e9 / PEAK_HBM_GBS for k in stages}},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and B == 1:
         del xm, spec, out
         res["cpu_baseline"] = cpu_baseline_spectral_block(nlat, nlon, L, M, "legendre-gauss", C, conv.weight)
     return res
@@ -755,8 +764,8 @@ def legendre_fp32_mfma_figure(iters=10):
     sp = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
-    xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
-    spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
+    xm = torch.empty(lib.sfno_fourier_elems(pf, R), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, R), dtype=torch.float32, device=dev)
     check(lib.sfno_rfft(pf, P(x), 0, P(xm), C, sp), "rfft")
     ana = event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream)
     syn = event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream)

@@ -71,12 +71,13 @@ extern "C" {
 #define SFNO_DTYPE_BF16 1
 
 /* arithmetic of the Legendre / channel-mix contractions */
-#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  The channel mix runs them on the fp16 matrix pipe: each
-                                  * operand row is scaled by a power of two and cut into two fp16 numbers (22 of its 24
-                                  * significant bits), three products per term are accumulated in fp32 and the scales are
-                                  * undone on output (error of the size of fp32 rounding, relative to |x||w| summed
-                                  * over the row).  The Legendre stage uses three exact bf16 parts per operand and six
-                                  * products.  Channel mixes with an odd number of input channels run on fp32 MFMA. */
+#define SFNO_COMPUTE_FP32 0      /* fp32 operands, fp32 accumulate.  Both contractions (Legendre stage and channel mix) run on
+                                  * the fp16 matrix pipe: each operand is scaled by a power of two (tables and weights per
+                                  * row or column when they are packed, activations per row or per panel column as they are
+                                  * staged) and cut into two fp16 numbers (22 of its 24 significant bits), three of the four
+                                  * partial products are accumulated in fp32 and the scales are undone on output: error of
+                                  * the size of fp32 rounding, relative to the sum of |x||t| over the contracted index.
+                                  * Channel mixes with an odd number of input channels run on fp32 MFMA. */
 #define SFNO_COMPUTE_BF16 1      /* bf16 MFMA inputs (tables and activations rounded to bf16), fp32 accumulate */
 #define SFNO_COMPUTE_FP32_MFMA 2 /* transform plans only: as SFNO_COMPUTE_FP32 with the Legendre stage on the fp32 MFMA
                                   * instruction (fp32 tables, no operand splitting) */

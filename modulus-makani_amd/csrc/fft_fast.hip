@@ -205,17 +205,19 @@ __device__ __forceinline__ float4 widen4(uint2 v) {
 __device__ __forceinline__ void use_here(float4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 __device__ __forceinline__ void use_here(uint2& v) { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
 
-__device__ __forceinline__ unsigned bf16_rne(float f) {
-    unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;      // NaN stays NaN
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+// two floats rounded to nearest-even bf16 in one word (the hardware conversion: one instruction per pair, NaN stays NaN)
+__device__ __forceinline__ unsigned bf16_pair(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 f = {lo, hi};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
 }
 template <bool BF16>
 __device__ __forceinline__ void store4(void* base, int64_t idx, float4 v) {
     if (BF16) {
         uint2 o;
-        o.x = bf16_rne(v.x) | (bf16_rne(v.y) << 16);
-        o.y = bf16_rne(v.z) | (bf16_rne(v.w) << 16);
+        o.x = bf16_pair(v.x, v.y);
+        o.y = bf16_pair(v.z, v.w);
         *reinterpret_cast<uint2*>(reinterpret_cast<unsigned short*>(base) + idx) = o;
     } else {
         *reinterpret_cast<float4*>(reinterpret_cast<float*>(base) + idx) = v;

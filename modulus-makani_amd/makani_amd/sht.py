@@ -97,8 +97,9 @@ class _SHTBase(nn.Module):
     def __init__(self, nlat, nlon, lmax=None, mmax=None, grid="lobatto", norm="ortho", csphase=True, compute="fp32"):
         super().__init__()
         # compute = "fp32" (default, the reference's arithmetic): fp32 operands and accumulation, the Legendre stage on the
-        #   bf16 matrix pipe with every operand cut exactly into three bf16 numbers;
-        # "fp32_mfma": the same on the fp32 matrix instruction;
+        #   fp16 matrix pipe with every operand scaled by a power of two and cut into two fp16 numbers (three products);
+        # "fp32_bf16x3": every operand cut exactly into three bf16 numbers (six products, no scales);
+        # "fp32_mfma": the fp32 matrix instruction on fp32 tables;
         # "bf16": bf16 tables and inputs, fp32 accumulation.
         if compute not in ("fp32", "bf16", "fp32_mfma", "fp32_bf16x3"):
             raise ValueError(f"unknown compute mode {compute!r}, expected 'fp32', 'fp32_mfma', 'fp32_bf16x3' or 'bf16'")

@@ -764,8 +764,8 @@ def legendre_fp32_mfma_figure(iters=10):
     sp = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     pf, pi = sht.plan(dev).handle, isht.plan(dev).handle
-    xm = torch.empty(lib.sfno_fourier_elems(pf, R), dtype=torch.float32, device=dev)
-    spec = torch.empty(lib.sfno_spectral_elems(pf, R), dtype=torch.float32, device=dev)
+    xm = torch.empty(lib.sfno_fourier_elems(pf, C), dtype=torch.float32, device=dev)
+    spec = torch.empty(lib.sfno_spectral_elems(pf, C), dtype=torch.float32, device=dev)
     check(lib.sfno_rfft(pf, P(x), 0, P(xm), C, sp), "rfft")
     ana = event_time_ms(lambda: check(lib.sfno_legendre_analysis(pf, P(xm), P(spec), C, sp), "analysis"), iters, stream)
     syn = event_time_ms(lambda: check(lib.sfno_legendre_synthesis(pi, P(spec), P(xm), C, sp), "synthesis"), iters, stream)

@@ -303,6 +303,18 @@ int sfno_pointwise_conv(const void* x, const void* w, const float* bias, void* y
 int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, int K2, const void* w, const float* bias, void* y,
                             int batch, int O, int64_t P, int act, void* stream);
 
+/* Gradients of that convolution with respect to its parameters, for training through it (what autograd derives for
+ * nn.Conv2d(kernel_size=1), makani/models/common/layers.py:95-116,160-216; the reference trains the whole block,
+ * makani/models/networks/sfnonet.py:239-267):
+ *   gweight[o][k] = sum_{b,p} gy[b][o][p] x[b][k][p],      gbias[o] = sum_{b,p} gy[b][o][p]
+ * gy bf16 [B][O][P], x bf16 [B][K][P] (both 16-byte aligned, P a multiple of 8); gweight float32 [O][K]; gbias float32 [O]
+ * or null.  fp32 accumulation in a fixed order (bit-identical from call to call).  `workspace` holds
+ * sfno_pointwise_weight_grad_workspace_bytes(batch, K, O, P, gbias != null) bytes.  The gradient with respect to the
+ * input is sfno_pointwise_conv itself on gy with the transposed weight ([K][O]) packed. */
+size_t sfno_pointwise_weight_grad_workspace_bytes(int batch, int K, int O, int64_t P, int has_bias);
+int sfno_pointwise_weight_grad(const void* gy, const void* x, float* gweight, float* gbias, int batch, int K, int O,
+                               int64_t P, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Packs a 1x1 convolution weight (float32 [O][K], the nn.Conv2d parameter viewed as a matrix) into the bf16
  * MFMA operand stream sfno_pointwise_conv reads; `packed` holds sfno_pointwise_weight_elems(O, K) bf16 values. */
 int64_t sfno_pointwise_weight_elems(int O, int K);

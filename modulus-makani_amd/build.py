@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 OUT = os.path.join(HERE, "makani_amd", "libsfno_spectral.so")
-SOURCES = ["tables.cpp", "capi.cpp", "dhconv.hip", "dhconv_f16.hip", "dhconv_wgrad.hip", "pointwise.hip", "diagonal.hip", "degree_power.hip", "legendre_fold.hip", "legendre_f16.hip", "fft.hip",
+SOURCES = ["tables.cpp", "capi.cpp", "dhconv.hip", "dhconv_f16.hip", "dhconv_wgrad.hip", "pointwise.hip", "pointwise_wgrad.hip", "diagonal.hip", "degree_power.hip", "legendre_fold.hip", "legendre_f16.hip", "fft.hip",
            "fft_fast.hip", "layout.hip", "static_scratch.hip"]
 HEADERS = [os.path.join(CSRC, "sfno_internal.h"), os.path.join(CSRC, "dhconv_map.h"), os.path.join(ROOT, "include", "sfno_spectral.h")]
 

@@ -615,6 +615,20 @@ extern "C" int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, i
     return pointwise_gemm_launch(a, (hipStream_t)stream);
 }
 
+extern "C" size_t sfno_pointwise_weight_grad_workspace_bytes(int batch, int K, int O, int64_t P, int has_bias) {
+    if (batch < 1 || K < 1 || O < 1 || P < 8 || P % 8) return 0;
+    return pointwise_wgrad_workspace_bytes(O, K, has_bias, batch, P);
+}
+
+extern "C" int sfno_pointwise_weight_grad(const void* gy, const void* x, float* gweight, float* gbias, int batch, int K, int O, int64_t P,
+                                          void* workspace, size_t workspace_bytes, void* stream) {
+    if (!gy || !x || !gweight || !workspace || batch < 1 || K < 1 || O < 1 || P < 8 || P % 8) return SFNO_EINVAL;
+    // 16-byte loads of eight bf16 values
+    if ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(x)) & 15) return SFNO_EINVAL;
+    return pointwise_wgrad_launch(reinterpret_cast<const unsigned short*>(gy), reinterpret_cast<const unsigned short*>(x), gweight, gbias, batch, K, O, P,
+                                  reinterpret_cast<float*>(workspace), workspace_bytes, (hipStream_t)stream);
+}
+
 extern "C" size_t sfno_instance_norm_workspace_bytes(int64_t rows, int64_t P) {
     if (rows < 1 || P < 1) return 0;
     return sizeof(float2) * (size_t)rows * row_stats_segments(rows, P);

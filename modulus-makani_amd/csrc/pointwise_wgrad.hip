@@ -1,0 +1,235 @@
+// Weight gradient of the 1x1 convolution on bf16 NCHW activations:
+//
+//   dW[o][k] = sum_{b,p} g[b][o][p] x[b][k][p],      db[o] = sum_{b,p} g[b][o][p]
+//
+// (what autograd derives for nn.Conv2d(kernel_size=1), makani/models/common/layers.py:95-116,160-216).  Both operands are
+// pixel-contiguous and the sum runs over the pixels, so a row of g is an A operand and a row of x a B operand of
+// v_mfma_f32_32x32x16_bf16 as they lie in memory: 8 consecutive pixels per lane, no transposition.  The bias gradient
+// rides along as one more column: row K of x is taken to be all ones.
+//
+// A workgroup (four wavefronts, 2 x 2) owns a 128 x 256 tile of dW and a contiguous share of the (sample, 32-pixel chunk)
+// sequence.  Per chunk 128 rows of g and 256 rows of x (64 bytes each) go straight from memory into a ring of three LDS
+// stages with global_load_lds_dwordx4, two chunks ahead of the matrix instructions (issued from inline assembly with a
+// counted wait, as in the forward kernel); a lane fetches the 16-byte piece whose LDS slot it owns, and the pieces of a row
+// are permuted by (row >> 1) & 3 so that the 16-byte fragment reads of eight consecutive rows cover all banks.  Pieces
+// past the end of a sample come from a block of zeros, the bias column from a block of ones.  Each wavefront multiplies
+// 64 x 128 (two A and four B fragments per 16 pixels for eight matrix instructions).  The shares' partial tiles go to a
+// workspace [share][O][K + 1] and a second kernel adds them up in a fixed order: results do not depend on scheduling.
+// All tiles of one share run on one XCD (workgroups are dealt to the XCDs round robin by linear id), where they meet
+// the share's rows of g and x in L2.
+#include "sfno_internal.h"
+
+namespace sfno {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WG_TO = 128;            // rows of dW (output channels) per workgroup
+constexpr int WG_TK = 256;            // columns of dW (input channels, + the bias column) per workgroup
+constexpr int WG_PX = 32;             // pixels per chunk: four 16-byte pieces per row
+constexpr int WG_ROWS = WG_TO + WG_TK;
+constexpr int WG_STAGE = WG_ROWS * 2 * WG_PX;                 // bytes per LDS stage
+constexpr int WG_STAGES = 3;
+constexpr int WG_PIECES = WG_ROWS * (WG_PX / 8) / 256;        // 16-byte pieces per thread and chunk
+static_assert(WG_PX == 32, "four pieces per row: the permutation and the slot arithmetic below");
+static_assert(WG_ROWS * (WG_PX / 8) % 256 == 0, "the chunk divides evenly among the threads");
+static_assert(WG_TO * (WG_PX / 8) % 256 == 0, "a thread's piece j is a row of g for all threads or a row of x for all threads");
+
+// sources of the pieces that are not read from the tensors
+__device__ __align__(16) const unsigned int wg_zero16[4] = {0u, 0u, 0u, 0u};
+__device__ __align__(16) const unsigned int wg_ones16[4] = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+
+// 16 bytes per lane from global memory to LDS base + 16 lane (M0 carries the base; the compiler reserves M0 and does not
+// accept it on a clobber list: nothing else in this file may depend on M0)
+__device__ __forceinline__ void wg_dma16(const void* g, unsigned lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte_addr) : "memory");
+}
+
+struct WgradShape {
+    int n_ot, n_kt, splits;
+    int64_t cps, chunks;               // chunks per sample, chunks in all
+};
+
+// how the launcher and the workspace query divide the work: shares of at least eight chunks, some two workgroups per CU
+static WgradShape wgrad_shape(int O, int Kext, int B, int64_t P) {
+    WgradShape s;
+    s.n_ot = (O + WG_TO - 1) / WG_TO;
+    s.n_kt = (Kext + WG_TK - 1) / WG_TK;
+    s.cps = (P + WG_PX - 1) / WG_PX;
+    s.chunks = s.cps * B;
+    const int tiles = s.n_ot * s.n_kt;
+    int64_t want = (512 + tiles - 1) / tiles;
+    want = (want + 7) / 8 * 8;
+    const int64_t most = (s.chunks + 7) / 8;       // at least eight chunks per share
+    if (want > most) want = most;
+    if (want < 1) want = 1;
+    s.splits = (int)want;
+    return s;
+}
+
+struct WgradArgs {
+    const unsigned short* G;           // bf16 [B][O][P]
+    const unsigned short* X;           // bf16 [B][K][P]
+    float* ws;                         // [splits][O][Kext]
+    int O, K, Kext, B;
+    int64_t P;
+    int n_ot, n_kt, splits;
+    int64_t cps, chunks;
+};
+
+// grid = 8 * ceil(splits / 8) * n_ot * n_kt workgroups of 256 threads
+__global__ __launch_bounds__(256, 2) void pw_wgrad_kernel(WgradArgs a) {
+    __shared__ __align__(16) unsigned char lds[WG_STAGES * WG_STAGE];
+    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+    const int tiles = a.n_ot * a.n_kt;
+    const int split = (q / tiles) * 8 + xcd, tile = q % tiles;
+    if (split >= a.splits) return;
+    const int o0 = (tile % a.n_ot) * WG_TO, k0 = (tile / a.n_ot) * WG_TK;
+    const int64_t c_begin = (int64_t)split * a.chunks / a.splits, c_end = (int64_t)(split + 1) * a.chunks / a.splits;
+    const int nch = (int)(c_end - c_begin);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wo = wave & 1, wk = wave >> 1;
+    const unsigned lds0 = (unsigned)(size_t)((__attribute__((address_space(3))) unsigned char*)lds);
+
+    // ---- loads: LDS slot s = 256 j + tid of a stage (16 bytes) holds row s >> 2, piece (s & 3) ^ ((row >> 1) & 3); rows below
+    // WG_TO are rows of g, the others rows of x.  A thread's six slots lie 64 rows apart: same piece, same permutation.
+    constexpr int JG = WG_TO * (WG_PX / 8) / 256;
+    const int part = (tid & 3) ^ ((tid >> 3) & 3);
+    const unsigned short* rowp[WG_PIECES];     // first pixel of the row in sample 0 (rows past the matrix: its last row, whose products are never stored)
+    bool ones[WG_PIECES];                      // the bias column: all ones
+#pragma unroll
+    for (int j = 0; j < WG_PIECES; ++j) {
+        const int row = (tid >> 2) + 64 * j;
+        if (j < JG) {
+            rowp[j] = a.G + (int64_t)min(o0 + row, a.O - 1) * a.P;
+            ones[j] = false;
+        } else {
+            const int k = k0 + row - WG_TO;
+            rowp[j] = a.X + (int64_t)min(k, a.K - 1) * a.P;
+            ones[j] = k == a.K && a.Kext > a.K;
+        }
+    }
+    const unsigned short* zero16 = reinterpret_cast<const unsigned short*>(wg_zero16);
+    const unsigned short* ones16 = reinterpret_cast<const unsigned short*>(wg_ones16);
+    // next chunk to ask for: sample ib, chunk ic of the sample (counted along: no division per chunk)
+    int64_t ib = c_begin / a.cps;
+    int64_t ic = c_begin - ib * a.cps;
+    auto issue = [&](int stage) {
+        const int64_t p = ic * WG_PX + 8 * part;
+        const bool in = p < a.P;               // P is a multiple of 8: a piece lies inside the row or outside
+        const int64_t og = ib * a.O * a.P + p, ox = ib * a.K * a.P + p;
+        const unsigned dst = lds0 + stage * WG_STAGE + wave * 1024;
+#pragma unroll
+        for (int j = 0; j < WG_PIECES; ++j) {
+            const unsigned short* src = !in ? zero16 : ones[j] ? ones16 : rowp[j] + (j < JG ? og : ox);
+            wg_dma16(src, dst + j * 4096);
+        }
+        if (++ic == a.cps) {
+            ic = 0;
+            ++ib;
+        }
+    };
+
+    f32x16 acc[2][4];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.f;
+
+    // fragments of this lane: row (lane & 31) of a 32-row block, pieces (lane >> 5) and 2 + (lane >> 5) of the row (pixels
+    // 8 (lane >> 5) .. + 7 of the first and of the second 16-pixel step), at their permuted places
+    const int sw = (lane >> 1) & 3, kg = lane >> 5;
+    const unsigned fa = (wo * 64 + (lane & 31)) * 64, fb = (WG_TO + wk * 128 + (lane & 31)) * 64;
+    const unsigned pk[2] = {(unsigned)((kg ^ sw) * 16), (unsigned)(((2 + kg) ^ sw) * 16)};
+
+    // Ring of three stages: chunk i is multiplied while chunks i + 1 and i + 2 are on their way.  The only vector memory
+    // operations of the loop are the six loads per wavefront and chunk, so "at most six outstanding" means chunk i has landed.
+    if (nch > 0) issue(0);
+    if (nch > 1) issue(1);
+    int stage = 0;
+    for (int i = 0; i < nch; ++i) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + 1 < nch)
+            asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // (every wavefront has read chunk i - 1: its stage takes chunk i + 2)
+        if (i + 2 < nch) issue(stage == 0 ? 2 : stage - 1);
+        const unsigned char* sb = lds + stage * WG_STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            bf16x8 af[2], bf[4];
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) af[mt] = *reinterpret_cast<const bf16x8*>(sb + fa + mt * 32 * 64 + pk[ks]);
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) bf[nt] = *reinterpret_cast<const bf16x8*>(sb + fb + nt * 32 * 64 + pk[ks]);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt], bf[nt], acc[mt][nt], 0, 0, 0);
+        }
+        stage = stage == 2 ? 0 : stage + 1;
+    }
+
+    // D layout of the 32x32 MFMA: register v of lane j holds D[8 (v / 4) + 4 (j / 32) + v % 4][j % 32]
+    float* out = a.ws + (int64_t)split * a.O * a.Kext;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            const int kk = k0 + wk * 128 + nt * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int o = o0 + wo * 64 + mt * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (o < a.O && kk < a.Kext) out[(int64_t)o * a.Kext + kk] = acc[mt][nt][v];
+            }
+        }
+}
+
+// dW[o][k] = sum over the shares, in order; column K goes to db
+__global__ __launch_bounds__(256) void pw_wgrad_reduce_kernel(const float* __restrict__ ws, float* __restrict__ dW, float* __restrict__ db, int O, int K,
+                                                              int Kext, int splits) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)O * Kext) return;
+    const int o = (int)(idx / Kext), k = (int)(idx - (int64_t)o * Kext);
+    float s = 0.f;
+    for (int i = 0; i < splits; ++i) s += ws[(int64_t)i * O * Kext + idx];
+    if (k < K)
+        dW[(int64_t)o * K + k] = s;
+    else if (db)
+        db[o] = s;
+}
+
+size_t pointwise_wgrad_workspace_bytes(int O, int K, int has_bias, int B, int64_t P) {
+    const int Kext = K + (has_bias ? 1 : 0);
+    const WgradShape s = wgrad_shape(O, Kext, B, P);
+    return sizeof(float) * (size_t)s.splits * (size_t)O * (size_t)Kext;
+}
+
+int pointwise_wgrad_launch(const unsigned short* g, const unsigned short* x, float* dW, float* db, int B, int K, int O, int64_t P, float* ws,
+                           size_t ws_bytes, hipStream_t s) {
+    if (P < 8 || P % 8) return SFNO_EINVAL;
+    const int Kext = K + (db ? 1 : 0);
+    const WgradShape sh = wgrad_shape(O, Kext, B, P);
+    if (ws_bytes < sizeof(float) * (size_t)sh.splits * (size_t)O * (size_t)Kext) return SFNO_EINVAL;
+    WgradArgs a;
+    a.G = g; a.X = x; a.ws = ws;
+    a.O = O; a.K = K; a.Kext = Kext; a.B = B; a.P = P;
+    a.n_ot = sh.n_ot; a.n_kt = sh.n_kt; a.splits = sh.splits; a.cps = sh.cps; a.chunks = sh.chunks;
+    const int64_t nwg = 8 * (int64_t)((sh.splits + 7) / 8) * sh.n_ot * sh.n_kt;
+    if (nwg > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(pw_wgrad_kernel, dim3((unsigned)nwg), dim3(256), 0, s, a);
+    if (hipGetLastError() != hipSuccess) return SFNO_EHIP;
+    const int64_t n = (int64_t)O * Kext;
+    hipLaunchKernelGGL(pw_wgrad_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, ws, dW, db, O, K, Kext, sh.splits);
+    return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
+}
+
+}  // namespace sfno

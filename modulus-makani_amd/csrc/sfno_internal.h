@@ -100,6 +100,10 @@ int pointwise_gemm_launch(PointwiseArgs a, hipStream_t s);
 int pointwise_kpad(int K, int O);
 int pointwise_opad(int O);
 int pointwise_pack_launch(const float* w, unsigned short* packed, int O, int K, hipStream_t s);
+// weight and bias gradient of the 1x1 convolution (pointwise_wgrad.hip); db null: no bias column
+size_t pointwise_wgrad_workspace_bytes(int O, int K, int has_bias, int B, int64_t P);
+int pointwise_wgrad_launch(const unsigned short* g, const unsigned short* x, float* dW, float* db, int B, int K, int O, int64_t P, float* ws,
+                           size_t ws_bytes, hipStream_t s);
 int row_stats_segments(int64_t rows, int64_t P);
 int instance_norm_coeffs_launch(const unsigned short* x, const float* gamma, const float* beta, float* scale, float* shift, float2* partial,
                                 int64_t rows, int channels, int64_t P, float eps, hipStream_t s);

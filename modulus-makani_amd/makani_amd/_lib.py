@@ -78,6 +78,8 @@ def _load():
         "sfno_pointwise_pack_weight": (i32, [vp, vp, i32, i32, vp]),
         "sfno_pointwise_conv": (i32, [vp, vp, vp, vp, i32, i32, i32, i64, i32, vp, vp, vp, vp]),
         "sfno_pointwise_conv_cat": (i32, [vp, i32, vp, i32, vp, vp, vp, i32, i32, i64, i32, vp]),
+        "sfno_pointwise_weight_grad_workspace_bytes": (sz, [i32, i32, i32, i64, i32]),
+        "sfno_pointwise_weight_grad": (i32, [vp, vp, vp, vp, i32, i32, i32, i64, vp, sz, vp]),
         "sfno_instance_norm_workspace_bytes": (sz, [i64, i64]),
         "sfno_instance_norm_coeffs": (i32, [vp, vp, vp, vp, vp, i64, i32, i64, c.c_float, vp, sz, vp]),
         "sfno_instance_norm_coeffs_lat": (i32, [vp, vp, vp, vp, vp, i64, i32, i32, c.c_float, vp]),

@@ -4,7 +4,9 @@
 instance norm split into its statistics (a per-(b, c) scale and shift) and their application.
 These replace the nn.Conv2d(kernel_size=1) / nn.InstanceNorm2d / nn.GELU sequences of
 makani/models/networks/sfnonet.py:246-262 and makani/models/common/layers.py:86-216 on the
-inference path under bf16 autocast; there is no backward through them.
+inference path under bf16 autocast.  The plain convolution (with its bias) also has a backward on the HIP
+kernels -- conv1x1_trainable, the forward of PointwiseConv2d when a gradient is asked for --, so that training under
+bf16 autocast keeps its 1x1 convolutions here; the fused epilogues have none.
 """
 import ctypes
 import weakref
@@ -155,3 +157,78 @@ def scale_shift_act(x, scale, shift, act=None):
     y = torch.empty_like(x)
     check(lib.sfno_scale_shift_act(_ptr(x), _ptr(scale), _ptr(shift), _ptr(y), B * C, H * W, ACT[act], _stream(x.device)), "sfno_scale_shift_act")
     return y
+
+
+def conv1x1_weight_grad(gy, x, with_bias):
+    """(gweight float32 [O, K], gbias float32 [O] or None) of y = conv1x1(x, weight) + bias for the output gradient gy:
+    gweight[o, k] = sum_{b,p} gy[b, o, p] x[b, k, p], gbias[o] = sum_{b,p} gy[b, o, p]; bf16 operands, fp32 sums in a fixed order."""
+    if not (supported(x) and supported(gy)) or gy.shape[0] != x.shape[0] or gy.shape[2:] != x.shape[2:]:
+        raise RuntimeError("conv1x1_weight_grad takes two contiguous bfloat16 NCHW HIP tensors of one batch and grid size, H*W a multiple of 8")
+    x, gy = x.contiguous(), gy.contiguous()
+    B, K, H, W = x.shape
+    O = gy.shape[1]
+    gw = torch.empty((O, K), dtype=torch.float32, device=x.device)
+    gb = torch.empty((O,), dtype=torch.float32, device=x.device) if with_bias else None
+    nbytes = lib.sfno_pointwise_weight_grad_workspace_bytes(B, K, O, H * W, 1 if with_bias else 0)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    check(lib.sfno_pointwise_weight_grad(_ptr(gy), _ptr(x), _ptr(gw), _ptr(gb), B, K, O, H * W, _ptr(ws), nbytes, _stream(x.device)),
+          "sfno_pointwise_weight_grad")
+    return gw, gb
+
+
+class _Conv1x1(torch.autograd.Function):
+    """y = conv1x1(x, weight) + bias on the HIP kernels, with the three gradients autograd derives for nn.Conv2d(kernel_size=1)
+    (makani/models/common/layers.py:95-116,160-216): the input gradient is the same convolution with the transposed weight."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        xb = x.detach().to(torch.bfloat16).contiguous()
+        ctx.save_for_backward(xb, weight)
+        ctx.has_bias = bias is not None
+        ctx.x_dtype = x.dtype
+        ctx.b_dtype = bias.dtype if bias is not None else None
+        # (the parameter itself goes in: its packed copy is cached per parameter object and version)
+        return conv1x1(xb, weight, bias)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gy):
+        xb, weight = ctx.saved_tensors
+        gy = gy.to(torch.bfloat16).contiguous()
+        gx = gw = gb = None
+        if ctx.needs_input_grad[0]:
+            wt = weight.detach().reshape(weight.shape[0], -1).t().contiguous()       # [K, O]: packed afresh, it is no parameter
+            gx = conv1x1(gy, wt).to(ctx.x_dtype)
+        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+            gw, gb = conv1x1_weight_grad(gy, xb, ctx.has_bias)
+            gw = gw.reshape(weight.shape).to(weight.dtype)
+            if gb is not None:
+                gb = gb.to(ctx.b_dtype)
+        return gx, gw, gb
+
+
+def trainable_active(x):
+    """Whether PointwiseConv2d routes this call through the HIP kernels: a gradient is being recorded and the activations are
+    bf16 (or will be under bf16 autocast) HIP tensors the kernels take."""
+    if not torch.is_grad_enabled() or not x.is_cuda or x.dim() != 4:
+        return False
+    bf16 = x.dtype == torch.bfloat16 or (torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16)
+    return bf16 and (x.shape[2] * x.shape[3]) % 8 == 0 and x.shape[2] * x.shape[3] >= 8
+
+
+def conv1x1_trainable(x, weight, bias=None):
+    """conv1x1(x, weight) + bias -> bf16, differentiable with respect to x, weight and bias (HIP kernels in both directions)."""
+    return _Conv1x1.apply(x, weight, bias)
+
+
+class PointwiseConv2d(torch.nn.Conv2d):
+    """nn.Conv2d(kernel_size=1) whose training forward and backward under bf16 run on the HIP kernels; every other call (fp32,
+    CPU, no gradient) is nn.Conv2d.  Same parameters and state-dict keys."""
+
+    def __init__(self, in_channels, out_channels, bias=True):
+        super().__init__(in_channels, out_channels, 1, bias=bias)
+
+    def forward(self, x):
+        if trainable_active(x) and (x.requires_grad or self.weight.requires_grad):
+            return conv1x1_trainable(x, self.weight, self.bias)
+        return super().forward(x)

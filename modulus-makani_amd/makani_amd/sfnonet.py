@@ -81,7 +81,7 @@ def fused_pointwise_active(x):
 
 
 def _pointwise(cin, cout, bias, std):
-    conv = nn.Conv2d(cin, cout, 1, bias=bias)
+    conv = pw.PointwiseConv2d(cin, cout, bias=bias)
     nn.init.normal_(conv.weight, mean=0.0, std=std)
     if bias:
         nn.init.constant_(conv.bias, 0.0)

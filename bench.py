@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SFNO spectral hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block|sfno8l|rollout|fft2_pair]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block|sfno8l|rollout|fft2_pair|pointwise_backward]
 
 Default workload (the configuration the headline metric is quoted on): forward + inverse
 real SHT at 721x1440 (equiangular, lmax = mmax = 721), batch 1, 73 channels, float32,
@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair"])
+    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair", "pointwise_backward"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--compute", default="fp32", choices=["fp32", "fp32_bf16x3", "bf16", "fp32_mfma"],
                     help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision: operands scaled and cut into two fp16 parts, "
@@ -748,6 +748,48 @@ def bench_rollout(args):
     }
 
 
+def bench_pointwise_backward(args):
+    """Backward of the 1x1 convolutions of the SFNO-8L tail at their in-model shapes (bf16): weight + bias gradient and input
+    gradient on the HIP kernels, with the kernels PyTorch picks for the same F.conv2d gradients beside them."""
+    import torch
+    import torch.nn.functional as F
+    from makani_amd import pointwise as pw
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev)
+    iters = max(args.steps, 5)
+    shapes = [("fc1 384->768 240x480", 384, 768, 240, 480), ("fc2 768->384 240x480", 768, 384, 240, 480), ("skip 384->384 240x480", 384, 384, 240, 480),
+              ("fc1 384->768 721x1440", 384, 768, 721, 1440), ("encoder 73->384 721x1440", 73, 384, 721, 1440), ("decoder 384->73 721x1440", 384, 73, 721, 1440)]
+    out, total = {}, 0.0
+    for name, K, O, H, W in shapes:
+        x = torch.randn(1, K, H, W, device=dev).bfloat16()
+        gy = torch.randn(1, O, H, W, device=dev).bfloat16()
+        w = torch.randn(O, K, 1, 1, device=dev) / K ** 0.5
+        wt = w.reshape(O, K).t().contiguous()
+        wb = w.bfloat16().requires_grad_(True)
+        xr = x.clone().requires_grad_(True)
+        y = F.conv2d(xr, wb)
+        for f in (lambda: pw.conv1x1_weight_grad(gy, x, True), lambda: pw.conv1x1(gy, wt)):
+            for _ in range(3):
+                f()
+        t_w = event_time_ms(lambda: pw.conv1x1_weight_grad(gy, x, True), iters, stream)
+        t_x = event_time_ms(lambda: pw.conv1x1(gy, wt), iters, stream)
+        for _ in range(3):
+            torch.autograd.grad(y, (wb, xr), gy, retain_graph=True)
+        t_lw = event_time_ms(lambda: torch.autograd.grad(y, wb, gy, retain_graph=True), iters, stream)
+        t_lx = event_time_ms(lambda: torch.autograd.grad(y, xr, gy, retain_graph=True), iters, stream)
+        nbytes = 2.0 * H * W * (K + O)
+        out[name] = {"weight_grad_ms": t_w, "input_grad_ms": t_x, "weight_grad_frac_hbm": nbytes / (t_w * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                     "input_grad_frac_hbm": nbytes / (t_x * 1e-3) / 1e9 / PEAK_HBM_GBS, "library_weight_grad_ms": t_lw, "library_input_grad_ms": t_lx}
+        total += t_w + t_x
+        del x, gy, y, xr
+    return {"metric": "1x1 convolution backward, sum over the listed shapes", "value": total, "unit": "ms", "n_gpus": 1, "steps": iters, "warmup": 3,
+            "ms_per_step": total, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "weight/bias and input gradients of the SFNO-8L tail's 1x1 convolutions, batch 1, bf16, N(0,1) operands"},
+            "shapes": out}
+
+
 def legendre_fp32_mfma_figure(iters=10):
     """The Legendre stage of configs[1] on the fp32 matrix instruction (compute="fp32_mfma"): time per direction and algorithmic
     (triangular) flops over it against the fp32 MFMA peak."""
@@ -832,6 +874,8 @@ def main():
         res = bench_spectral_block(args)
     elif args.workload == "sfno8l":
         res = bench_sfno8l(args)
+    elif args.workload == "pointwise_backward":
+        res = bench_pointwise_backward(args)
     else:
         res = bench_rollout(args)
     print(json.dumps(res), flush=True)

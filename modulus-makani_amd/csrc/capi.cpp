@@ -28,6 +28,7 @@ void free_table(PgemmTable& t) {
     if (t.d_rinv) (void)hipFree(t.d_rinv);
     if (t.d_aoff) (void)hipFree(t.d_aoff);
     if (t.d_work) (void)hipFree(t.d_work);
+    if (t.d_wrec) (void)hipFree(t.d_wrec);
     t = PgemmTable();
 }
 
@@ -62,6 +63,29 @@ int build_legendre_table(const sfno_sht_plan& p, const double* theta, const doub
     if (p.format == PG_FORMAT_F16X2 && (rc = upload(&t.d_rinv, rinv)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_aoff, aoff)) != SFNO_OK) return rc;
     if ((rc = upload(&t.d_work, work)) != SFNO_OK) return rc;
+    if (p.format == PG_FORMAT_F16X2) {
+        std::vector<int64_t> wrec(work.size() * PG_WREC, 0);
+        for (size_t w = 0; w < work.size(); ++w) {
+            int64_t* r = &wrec[w * PG_WREC];
+            const int m = work[w].x, rb0 = work[w].y;
+            r[PG_WREC_M] = m;
+            r[PG_WREC_RB] = rb0;
+            if (m < 0) continue;
+            const int nl0 = (p.lmax - m > 0) ? (p.lmax - m + 1) / 2 : 0;
+            const int nl1 = (p.lmax - m - 1 > 0) ? (p.lmax - m) / 2 : 0;
+            const int nc = analysis ? (K2 + PG_KC - 1) / PG_KC : (nl0 + PG_KC - 1) / PG_KC;
+            for (int par = 0; par < 2; ++par) {
+                const int nr = analysis ? (par ? nl1 : nl0) : K2;
+                r[PG_WREC_POS + par] = aoff[2 * m + par];
+                for (int j = 0; j < 2; ++j) {
+                    const int rb = rb0 + j;
+                    // (an order without degrees has no entries: nc = 0; a row block past the stream's rows has none either)
+                    r[PG_WREC_ENTRY + 2 * par + j] = (nc > 0 && rb * PG_ROWS < nr) ? aoff[(size_t)(aoff[2 * m + par] + rb)] : (int64_t)nc << 48;
+                }
+            }
+        }
+        if ((rc = upload(&t.d_wrec, wrec)) != SFNO_OK) return rc;
+    }
     return SFNO_OK;
 }
 
@@ -88,6 +112,7 @@ PgemmArgs legendre_args(const sfno_sht_plan* p, const PgemmTable& t, const float
     a.A = t.d_A;
     a.a_off = t.d_aoff;
     a.work = t.d_work;
+    a.wrec = t.d_wrec;
     a.Q = q;
     a.Out = out;
     a.rinv = t.d_rinv;

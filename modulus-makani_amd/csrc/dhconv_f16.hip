@@ -230,10 +230,25 @@ __global__ __launch_bounds__(256, 2) void dhconv_f16_kernel(DhconvArgs a) {
 #pragma unroll
     for (int t = 0; t < NTC; ++t) cinv[t] = a.cinv[(int64_t)l * (a.nob * CO) + CO * ob + 32 * t + cl];
     const int Efinal = E;
+    const int nn0 = r0 + 32 * wave + 4 * kg;                       // my first row; the others are 8 (v / 4) + v % 4 further on
+    if (a.B == 1 && r0 + 32 * wave + 32 <= ncols && 2 * (CO * ob + CO) <= a.O2) {
+        // one sample and no row or channel of my tile outside the tensor: row = order, one address, constant steps
+        float* o = a.Y + ((int64_t)nn0 * a.L + l) * a.ld_out + 2 * (CO * ob + cl);
+        const int64_t rstep = (int64_t)a.L * a.ld_out;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int er = __builtin_amdgcn_ds_bpermute(4 * (8 * (v >> 2) + 4 * kg + (v & 3)), Efinal);
+            float* orow = o + (8 * (v >> 2) + (v & 3)) * rstep;
+#pragma unroll
+            for (int t = 0; t < NTC; ++t)
+                *reinterpret_cast<f2*>(orow + 64 * t) = f2{__builtin_ldexpf(yr[t][v], er - DHF_SH) * cinv[t], __builtin_ldexpf(yi[t][v], er - DHF_SH) * cinv[t]};
+        }
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int er = __builtin_amdgcn_ds_bpermute(4 * (8 * (v >> 2) + 4 * kg + (v & 3)), Efinal);
-        const int nn = r0 + 32 * wave + 8 * (v >> 2) + 4 * kg + (v & 3);
+        const int nn = nn0 + 8 * (v >> 2) + (v & 3);
         if (nn >= ncols) continue;
         const int m2 = nn / a.B, b2 = nn - m2 * a.B;
         float* orow = a.Y + ((int64_t)m2 * a.L + l) * a.ld_out + (int64_t)b2 * a.O2;

@@ -61,9 +61,15 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
     const int nct = (a.ld + TN - 1) / TN;
     const int qid = blockIdx.x >> 3;
     const int ct = qid % nct;
-    const int2 wi = a.work[(qid / nct) * 8 + (blockIdx.x & 7)];
-    const int m = wi.x;
+    // (the record is read through the scalar unit: one 64-byte request, wavefront-uniform)
+    const __attribute__((address_space(4))) int64_t* wrec =
+        reinterpret_cast<const __attribute__((address_space(4))) int64_t*>(reinterpret_cast<uintptr_t>(a.wrec)) + (int64_t)((qid / nct) * 8 + (blockIdx.x & 7)) * PG_WREC;
+    int64_t rec[PG_WREC];
+#pragma unroll
+    for (int i = 0; i < PG_WREC; ++i) rec[i] = wrec[i];
+    const int m = (int)rec[PG_WREC_M];
     if (m < 0) return;
+    const int2 wi = make_int2(m, (int)rec[PG_WREC_RB]);
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     // wavefront w runs on SIMD w; alternate which SIMDs get the (possibly absent) second row block
     // and the (one row shorter) odd parity from workgroup to workgroup
@@ -88,16 +94,13 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
     // towards the poles the table falls off like sin^m(theta)).  The K loop of the workgroup starts at the smallest such
     // count of its (up to) four row blocks; a wavefront joins in at its own.
     constexpr int APB = 128;               // 16-byte pieces per block: two planes x 64 lanes
-    auto entry_pos = [&](int p_, int rb_) { return a.a_off[2 * m + p_] + rb_; };
-    auto entry_of = [&](int p_, int rb_) {
-        const int nr = ANALYSIS ? (p_ ? nl1 : nl0) : K2;
-        // an order without degrees (synthesis with mmax > lmax: nc = 0) has no entries; its rows are zero-filled below
-        return (nc > 0 && rb_ * PG_ROWS < nr) ? a.a_off[entry_pos(p_, rb_)] : (int64_t)nc << 48;
-    };
+    // (the work record holds the entries of the four streams -- nc << 48 for one that does not exist: an order without
+    // degrees, synthesis with mmax > lmax, has none, its rows are zero-filled below -- and the parities' first positions)
+    auto entry_pos = [&](int p_, int rb_) { return (p_ ? rec[PG_WREC_POS + 1] : rec[PG_WREC_POS]) + rb_; };
     int cstart = nc;
 #pragma unroll
-    for (int s_ = 0; s_ < 4; ++s_) cstart = min(cstart, (int)(entry_of(s_ >> 1, wi.y + (s_ & 1)) >> 48));
-    const int64_t my_entry = entry_of(par, rb);
+    for (int s_ = 0; s_ < 4; ++s_) cstart = min(cstart, (int)(rec[PG_WREC_ENTRY + s_] >> 48));
+    const int64_t my_entry = par ? ((wslot & 1) ? rec[PG_WREC_ENTRY + 3] : rec[PG_WREC_ENTRY + 2]) : ((wslot & 1) ? rec[PG_WREC_ENTRY + 1] : rec[PG_WREC_ENTRY]);
     cstart = max(cstart, 0);
     const int c0w = min(max((int)(my_entry >> 48), 0), nc);   // nc for a wavefront without a row block or with nothing but negligible entries
     const f4* apv = reinterpret_cast<const f4*>(a.A) + ((c0w < nc ? my_entry & (((int64_t)1 << 48) - 1) : (int64_t)0) * APB + lane);
@@ -295,6 +298,17 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
     if (ANALYSIS) {
         if (!active) return;
         float* out = a.Out + (int64_t)m * lmax * ld;
+        if (PG_ROWS * (rb + 1) <= nrows && n0 + TN <= ld) {
+            // no row or column of my tile needs a check: one address per row, the tiles at constant offsets from it
+            float* o = out + (int64_t)(m + par + 2 * (PG_ROWS * rb + 4 * kg)) * ld + n0 + cl;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float* orow = o + (int64_t)(2 * (8 * (v >> 2) + (v & 3))) * ld;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) orow[32 * t] = acc[t][v];
+            }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -323,7 +337,16 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
                 for (int v = 0; v < 16; ++v) mine[v * 64] = acc[t][v];
             }
             __syncthreads();
-            if (active) {
+            if (whole) {
+                // one address per wavefront tile, rows at multiples of +-ld from it, no checks
+                float* o = out + (int64_t)(par ? nlat - 1 - k0 : k0) * ld + n0 + 32 * t + cl;
+                const int64_t rstep = par ? -(int64_t)ld : (int64_t)ld;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float other = theirs[v * 64];
+                    o[(8 * (v >> 2) + (v & 3)) * rstep] = par ? other - acc[t][v] : acc[t][v] + other;
+                }
+            } else if (active) {
                 const int n = n0 + 32 * t + cl;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
@@ -332,7 +355,7 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
                     // even parity: E + O to row k; odd parity: E - O to row k' (the equator row is its own mirror and has O = 0)
                     const float x = par ? other - acc[t][v] : acc[t][v] + other;
                     const int row = par ? nlat - 1 - k : k;
-                    if (whole || (k < K2 && n < ld && !(par && row == k))) out[(int64_t)row * ld + n] = x;
+                    if (k < K2 && n < ld && !(par && row == k)) out[(int64_t)row * ld + n] = x;
                 }
             }
         }
@@ -343,7 +366,7 @@ template <bool ANALYSIS>
 static int launch_f16(const PgemmArgs& a, int n_work, hipStream_t s) {
     const int64_t ncols = a.ld;
     if (n_work <= 0 || ncols <= 0) return SFNO_OK;
-    if (!a.rinv) return SFNO_EINVAL;
+    if (!a.rinv || !a.wrec) return SFNO_EINVAL;
     // the kernel addresses a panel (one order: nlat or lmax rows of ld floats) with 32-bit byte offsets
     if ((int64_t)(a.nlat > a.lmax ? a.nlat : a.lmax) * a.ld >= ((int64_t)1 << 30)) return SFNO_EUNSUPPORTED;
     // prefer the least padding, then the tile count listed first

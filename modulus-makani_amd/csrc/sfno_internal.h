@@ -21,11 +21,18 @@ constexpr int PG_KC = 16;          // K per block
 constexpr int PG_BLOCK_FLOATS = PG_ROWS * PG_KC;   // 512 floats = 2 KiB
 constexpr int PG_WAVES = 4;        // wavefronts (= row blocks) per workgroup
 
+// Work record of the two-part fp16 kernels, 8 x int64 per work-list entry: the order and first row block, the index
+// entries of the workgroup's four (parity, row block) streams (an absent one reads nc << 48: nothing to do) and the
+// positions of the two parities' first entries -- one 64-byte read instead of a chain of dependent look-ups.
+constexpr int PG_WREC = 8;
+constexpr int PG_WREC_M = 0, PG_WREC_RB = 1, PG_WREC_ENTRY = 2, PG_WREC_POS = 6;
+
 struct PgemmTable {
     float* d_A = nullptr;          // packed stream
     float* d_rinv = nullptr;       // two-part fp16 format: 32 factors per row-block entry that undo the row scales
     int64_t* d_aoff = nullptr;     // index of the stream, see pack_legendre_fold
     int2* d_work = nullptr;        // [n_work] {batch, first row block} per workgroup, -1 = idle
+    int64_t* d_wrec = nullptr;     // two-part fp16 format: [n_work][8] everything a workgroup needs of the index, see PG_WREC_*
     int n_work = 0;                // multiple of 8 (one queue per XCD, interleaved)
     int64_t n_blocks = 0;
 };
@@ -34,6 +41,7 @@ struct PgemmArgs {
     const float* A;
     const int64_t* a_off;
     const int2* work;
+    const int64_t* wrec;           // two-part fp16 format: work records (PG_WREC_*)
     const float* Q;
     float* Out;
     const float* rinv;             // two-part fp16 format: row factors, [entry position - 2 mmax][32]

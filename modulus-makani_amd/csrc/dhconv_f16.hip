@@ -245,6 +245,21 @@ __global__ __launch_bounds__(256, 2) void dhconv_f16_kernel(DhconvArgs a) {
         }
         return;
     }
+    if ((a.B & (a.B - 1)) == 0 && r0 + 32 * wave + 32 <= ncols && 2 * (CO * ob + CO) <= a.O2) {
+        // a power-of-two number of samples, whole tile inside: (order, sample) of a row by shift and mask, no checks
+        const int lb = 31 - __builtin_clz(a.B);
+        float* o = a.Y + (int64_t)l * a.ld_out + 2 * (CO * ob + cl);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int er = __builtin_amdgcn_ds_bpermute(4 * (8 * (v >> 2) + 4 * kg + (v & 3)), Efinal);
+            const int nn = nn0 + 8 * (v >> 2) + (v & 3);
+            float* orow = o + (int64_t)(nn >> lb) * a.L * a.ld_out + (int64_t)(nn & (a.B - 1)) * a.O2;
+#pragma unroll
+            for (int t = 0; t < NTC; ++t)
+                *reinterpret_cast<f2*>(orow + 64 * t) = f2{__builtin_ldexpf(yr[t][v], er - DHF_SH) * cinv[t], __builtin_ldexpf(yi[t][v], er - DHF_SH) * cinv[t]};
+        }
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int er = __builtin_amdgcn_ds_bpermute(4 * (8 * (v >> 2) + 4 * kg + (v & 3)), Efinal);

@@ -38,12 +38,12 @@ constexpr int LH_HEAD = 3;             // bits of headroom left when a column's 
 constexpr int LH_SH = LH_TOP + 127;    // scaled = x * 2^(SH - E), E = biased exponent bound of the column
 
 // resident workgroups per CU: set by the 16 NT accumulator registers and the staged rows held across the matrix phase
-constexpr int lh_occupancy(int nt) { return nt <= 4 ? 4 : 2; }
+constexpr int lh_occupancy(int nt, bool analysis) { return nt <= 4 ? 4 : analysis ? 2 : 3; }
 
 __device__ __forceinline__ unsigned int lh_pk(float a, float b) { return __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_pkrtz(a, b)); }
 
 template <int NT, bool ANALYSIS>
-__global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(PgemmArgs a) {
+__global__ __launch_bounds__(256, lh_occupancy(NT, ANALYSIS)) void legendre_f16_kernel(PgemmArgs a) {
     constexpr int TN = 32 * NT;            // columns per workgroup
     constexpr int QN = TN / 4;             // column quads
     constexpr int QW = QN / 4;             // column quads staged per wavefront
@@ -179,33 +179,42 @@ __global__ __launch_bounds__(256, lh_occupancy(NT)) void legendre_f16_kernel(Pge
     };
     auto q_store = [&](int buf, int c) {
         if (!stager) return;
-        float v0[RPT], v1[RPT];
         // chunks that touch neither end of the K range nor the column tail need no masks
         const bool plain = col_ok && (ANALYSIS ? (c + 1) * PG_KC < K2 : m + 2 * (c + 1) * PG_KC < lmax);
-        if (plain) {
+        if constexpr (ANALYSIS) {
+            // i = latitude k; panel 0 = X[k] + X[k'], panel 1 = X[k] - X[k']; the equator row is its own mirror
+            float v0[RPT], v1[RPT];
+            if (plain) {
 #pragma unroll
-            for (int rr = 0; rr < RPT; ++rr) {
-                v0[rr] = ANALYSIS ? q0[rr] + q1[rr] : q0[rr];
-                v1[rr] = ANALYSIS ? q0[rr] - q1[rr] : q1[rr];
-            }
-        } else {
+                for (int rr = 0; rr < RPT; ++rr) {
+                    v0[rr] = q0[rr] + q1[rr];
+                    v1[rr] = q0[rr] - q1[rr];
+                }
+            } else {
 #pragma unroll
-            for (int rr = 0; rr < RPT; ++rr) {
-                const int i = c * PG_KC + RPT * shalf + rr;
-                if (ANALYSIS) {
-                    // i = latitude k; panel 0 = X[k] + X[k'], panel 1 = X[k] - X[k']; the equator row is its own mirror
+                for (int rr = 0; rr < RPT; ++rr) {
+                    const int i = c * PG_KC + RPT * shalf + rr;
                     const bool ok = col_ok && i < K2, mirror = (nlat - 1 - i) != i;
                     v0[rr] = ok ? (mirror ? q0[rr] + q1[rr] : q0[rr]) : 0.f;
                     v1[rr] = ok && mirror ? q0[rr] - q1[rr] : 0.f;
-                } else {
-                    // i = index within a parity; panel 0 = degree m+2i, panel 1 = degree m+2i+1
-                    v0[rr] = (col_ok && m + 2 * i < lmax) ? q0[rr] : 0.f;
-                    v1[rr] = (col_ok && m + 2 * i + 1 < lmax) ? q1[rr] : 0.f;
                 }
             }
+            cut_store(planes + ((buf * 2 + 0) * 2) * PLANE, v0, E0);
+            cut_store(planes + ((buf * 2 + 1) * 2) * PLANE, v1, E1);
+        } else {
+            // i = index within a parity; panel 0 = degree m+2i, panel 1 = degree m+2i+1.  What lies outside is zeroed in place (the
+            // raw rows are not needed again), so that the common case carries no copies of the 32 values
+            if (!plain) {
+#pragma unroll
+                for (int rr = 0; rr < RPT; ++rr) {
+                    const int i = c * PG_KC + RPT * shalf + rr;
+                    q0[rr] = (col_ok && m + 2 * i < lmax) ? q0[rr] : 0.f;
+                    q1[rr] = (col_ok && m + 2 * i + 1 < lmax) ? q1[rr] : 0.f;
+                }
+            }
+            cut_store(planes + ((buf * 2 + 0) * 2) * PLANE, q0, E0);
+            cut_store(planes + ((buf * 2 + 1) * 2) * PLANE, q1, E1);
         }
-        cut_store(planes + ((buf * 2 + 0) * 2) * PLANE, v0, E0);
-        cut_store(planes + ((buf * 2 + 1) * 2) * PLANE, v1, E1);
         if (shalf == 0) {
             expo[buf][0][scol] = E0;
             expo[buf][1][scol] = E1;

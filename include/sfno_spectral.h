@@ -307,7 +307,7 @@ int sfno_pointwise_conv_cat(const void* x1, int K1, const void* x2, int K2, cons
  * nn.Conv2d(kernel_size=1), makani/models/common/layers.py:95-116,160-216; the reference trains the whole block,
  * makani/models/networks/sfnonet.py:239-267):
  *   gweight[o][k] = sum_{b,p} gy[b][o][p] x[b][k][p],      gbias[o] = sum_{b,p} gy[b][o][p]
- * gy bf16 [B][O][P], x bf16 [B][K][P] (both 16-byte aligned, P a multiple of 8); gweight float32 [O][K]; gbias float32 [O]
+ * gy bf16 [B][O][P], x bf16 [B][K][P] (both, and the workspace, 16-byte aligned; P a multiple of 8); gweight float32 [O][K]; gbias float32 [O]
  * or null.  fp32 accumulation in a fixed order (bit-identical from call to call).  `workspace` holds
  * sfno_pointwise_weight_grad_workspace_bytes(batch, K, O, P, gbias != null) bytes.  The gradient with respect to the
  * input is sfno_pointwise_conv itself on gy with the transposed weight ([K][O]) packed. */

@@ -649,7 +649,7 @@ extern "C" int sfno_pointwise_weight_grad(const void* gy, const void* x, float* 
                                           void* workspace, size_t workspace_bytes, void* stream) {
     if (!gy || !x || !gweight || !workspace || batch < 1 || K < 1 || O < 1 || P < 8 || P % 8) return SFNO_EINVAL;
     // 16-byte loads of eight bf16 values
-    if ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(x)) & 15) return SFNO_EINVAL;
+    if ((reinterpret_cast<uintptr_t>(gy) | reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(workspace)) & 15) return SFNO_EINVAL;
     return pointwise_wgrad_launch(reinterpret_cast<const unsigned short*>(gy), reinterpret_cast<const unsigned short*>(x), gweight, gbias, batch, K, O, P,
                                   reinterpret_cast<float*>(workspace), workspace_bytes, (hipStream_t)stream);
 }

@@ -219,18 +219,36 @@ __global__ __launch_bounds__(WG_THREADS, 2) void pw_wgrad_kernel(WgradArgs a) {
         }
 }
 
-// dW[o][k] = sum over the shares, in order; column K goes to db
+// dW[o][k] = sum over the shares, in order; column K goes to db.  A thread sums four consecutive entries of the
+// [O][Kext] matrices (16-byte loads, eight shares in flight) and stores them one by one: they may straddle a row.
 __global__ __launch_bounds__(256) void pw_wgrad_reduce_kernel(const float* __restrict__ ws, float* __restrict__ dW, float* __restrict__ db, int O, int K,
                                                               int Kext, int splits) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)O * Kext) return;
-    const int o = (int)(idx / Kext), k = (int)(idx - (int64_t)o * Kext);
-    float s = 0.f;
-    for (int i = 0; i < splits; ++i) s += ws[(int64_t)i * O * Kext + idx];
-    if (k < K)
-        dW[(int64_t)o * K + k] = s;
-    else if (db)
-        db[o] = s;
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int64_t n = (int64_t)O * Kext;
+    const int64_t idx = 4 * ((int64_t)blockIdx.x * blockDim.x + threadIdx.x);
+    if (idx >= n) return;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (idx + 4 <= n && n % 4 == 0) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+        for (int i = 0; i < splits; ++i) acc += *reinterpret_cast<const f32x4*>(ws + (int64_t)i * n + idx);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] = acc[e];
+    } else {
+        for (int i = 0; i < splits; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (idx + e < n) s[e] += ws[(int64_t)i * n + idx + e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (idx + e >= n) break;
+        const int o = (int)((idx + e) / Kext), k = (int)(idx + e - (int64_t)o * Kext);
+        if (k < K)
+            dW[(int64_t)o * K + k] = s[e];
+        else if (db)
+            db[o] = s[e];
+    }
 }
 
 size_t pointwise_wgrad_workspace_bytes(int O, int K, int has_bias, int B, int64_t P) {
@@ -254,7 +272,7 @@ int pointwise_wgrad_launch(const unsigned short* g, const unsigned short* x, flo
     hipLaunchKernelGGL(pw_wgrad_kernel, dim3((unsigned)nwg), dim3(WG_THREADS), 0, s, a);
     if (hipGetLastError() != hipSuccess) return SFNO_EHIP;
     const int64_t n = (int64_t)O * Kext;
-    hipLaunchKernelGGL(pw_wgrad_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, ws, dW, db, O, K, Kext, sh.splits);
+    hipLaunchKernelGGL(pw_wgrad_reduce_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, ws, dW, db, O, K, Kext, sh.splits);
     return hipGetLastError() == hipSuccess ? SFNO_OK : SFNO_EHIP;
 }
 

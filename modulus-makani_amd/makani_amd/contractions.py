@@ -253,6 +253,25 @@ def _contract_diagonal(ac: torch.Tensor, bc: torch.Tensor) -> torch.Tensor:
     return _DiagonalFn.apply(ac.contiguous(), bc.contiguous())
 
 
+def _as_complex_weight(b):
+    """A real weight as the complex one with zero imaginary part (differentiable: the gradient is the real part of the complex one's)."""
+    return torch.complex(b, torch.zeros_like(b))
+
+
+def _contract_diagonal_real(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """einsum("bixys,ioxy->boxys"): complex activations as float32 [..., 2], real weight (contractions.py:157-160)."""
+    if a.dim() != 5 or a.shape[-1] != 2 or b.is_complex():
+        raise RuntimeError(f"diagonal (real weight): shapes {tuple(a.shape)} and {tuple(b.shape)} do not match 'bixys,ioxy->boxys'")
+    return torch.view_as_real(_contract_diagonal(torch.view_as_complex(a.contiguous()), _as_complex_weight(b))).contiguous()
+
+
+def _contract_dhconv_real(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """einsum("bixys,iox->boxys"): complex activations as float32 [..., 2], real weight (contractions.py:163-166)."""
+    if a.dim() != 5 or a.shape[-1] != 2 or b.is_complex():
+        raise RuntimeError(f"dhconv (real weight): shapes {tuple(a.shape)} and {tuple(b.shape)} do not match 'bixys,iox->boxys'")
+    return torch.view_as_real(_contract_dhconv(torch.view_as_complex(a.contiguous()), _as_complex_weight(b))).contiguous()
+
+
 def _contract_dense(x, weight, separable=False, operator_type="diagonal", complex=True):
     """Mirror of _contract_dense_pytorch (factorizations.py:167-200).
 
@@ -260,11 +279,11 @@ def _contract_dense(x, weight, separable=False, operator_type="diagonal", comple
     contractions.py:139-154) name an output index that no input carries, so they cannot be evaluated there either."""
     if operator_type not in ("diagonal", "dhconv"):
         raise ValueError(f"unknown operator type {operator_type!r}, expected 'diagonal' or 'dhconv'")
-    if separable or not complex:
-        raise NotImplementedError("only the non-separable complex operators run on the HIP path")
+    if separable:
+        raise NotImplementedError("the separable operators are not provided (see above)")
     if operator_type == "diagonal":
-        return _contract_diagonal(x, weight)
-    return _contract_dhconv(x, weight)
+        return _contract_diagonal(x, weight) if complex else _contract_diagonal_real(x, weight)
+    return _contract_dhconv(x, weight) if complex else _contract_dhconv_real(x, weight)
 
 
 def get_contract_fun(weight, implementation="reconstructed", separable=False, operator_type="diagonal", complex=True):

@@ -202,3 +202,32 @@ def test_spectral_conv_empty_batch(lib_built, updown):
     y.sum().backward()
     assert tuple(xg.grad.shape) == tuple(xg.shape) and tuple(conv.weight.grad.shape) == tuple(conv.weight.shape)
     assert float(conv.weight.grad.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("operator_type", ["dhconv", "diagonal"])
+def test_real_weight_contractions_and_their_gradients(lib_built, operator_type):
+    """complex=False (contractions.py:157-166): activations as float32 [..., 2], real weights -- values and gradients against
+    float64 autograd of the reference's einsum strings."""
+    import makani_amd as ma
+
+    print(f"case real-weight contraction {operator_type}", flush=True)
+    torch.manual_seed(8)
+    B, I, O, L, M = 2, 6, 4, 9, 7
+    eq = "bixys,iox->boxys" if operator_type == "dhconv" else "bixys,ioxy->boxys"
+    a = torch.randn(B, I, L, M, 2)
+    w = torch.randn(*((I, O, L) if operator_type == "dhconv" else (I, O, L, M))) / np.sqrt(I)
+    g = torch.randn(B, O, L, M, 2)
+    ag, wg = a.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    f = ma.get_contract_fun(wg, implementation="factorized", separable=False, complex=False, operator_type=operator_type)
+    y = f(ag, wg)
+    assert y.dtype == torch.float32 and tuple(y.shape) == (B, O, L, M, 2) and y.is_contiguous()
+    y.backward(g.cuda())
+    torch.cuda.synchronize()
+    ar, wr = a.double().requires_grad_(True), w.double().requires_grad_(True)
+    yr = torch.einsum(eq, ar, wr)
+    yr.backward(g.double())
+    assert rel_l2(y.detach().cpu().numpy(), yr.detach().numpy()) < TOL
+    assert rel_l2(ag.grad.cpu().numpy(), ar.grad.numpy()) < TOL
+    assert wg.grad.dtype == torch.float32 and rel_l2(wg.grad.cpu().numpy(), wr.grad.numpy()) < TOL
+    with pytest.raises(NotImplementedError):
+        ma.get_contract_fun(wg, separable=True, complex=False, operator_type=operator_type)(ag, wg)

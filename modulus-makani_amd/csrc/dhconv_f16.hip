@@ -276,17 +276,27 @@ __global__ __launch_bounds__(256, 2) void dhconv_f16_kernel(DhconvArgs a) {
     }
 }
 
-// cmax[l][o] = largest |Re|, |Im| of w[.][o][l] over the input channels (adjoint: of w[o][.][l], w being [O][I][L])
+// cmax[l][o] = largest |Re|, |Im| of w[.][o][l] over the input channels (adjoint: of w[o][.][l], w being [O][I][L]).  A thread
+// takes DHF_CMAX_I input channels of one (o, l) and joins the others with an integer atomic maximum on the bit pattern (the
+// values are magnitudes: their order as unsigned integers is their order as floats, a NaN ranks above all and stays); cmax is
+// cleared by the kernel in front.  grid (ceil(O L / 256), ceil(I / DHF_CMAX_I))
+constexpr int DHF_CMAX_I = 16;
+__global__ __launch_bounds__(256) void dhconv_colmax_clear_kernel(float* __restrict__ cmax, int64_t n) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < n) cmax[idx] = 0.f;
+}
 __global__ __launch_bounds__(256) void dhconv_colmax_kernel(const float2* __restrict__ w, float* __restrict__ cmax, int I, int O, int L, int adjoint) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;     // o * L + l
     if (idx >= (int64_t)O * L) return;
     const int o = (int)(idx / L), l = (int)(idx - (int64_t)o * L);
+    const int i0 = blockIdx.y * DHF_CMAX_I, i1 = min(i0 + DHF_CMAX_I, I);
     float mx = 0.f;
-    for (int i = 0; i < I; ++i) {
+#pragma unroll 4
+    for (int i = i0; i < i1; ++i) {
         const float2 z = adjoint ? w[((int64_t)o * I + i) * L + l] : w[((int64_t)i * O + o) * L + l];
         mx = fmaxf(mx, fmaxf(fabsf(z.x), fabsf(z.y)));
     }
-    cmax[(int64_t)l * O + o] = mx;
+    atomicMax(reinterpret_cast<unsigned int*>(cmax) + ((int64_t)l * O + o), __float_as_uint(mx));
 }
 
 // Writes the stage images.  packed[l][ob][c] = [part (Re, Im)][plane][o (CO)][two 16-byte halves, see dhf_piece]: the half kg
@@ -360,7 +370,10 @@ int dhconv_pack_f16_launch(const float2* w, void* packed, float* cinv, float* cm
     if ((int64_t)nob * nc * ntc > 0x7fffffffLL || (L + 7) / 8 > 65535) return SFNO_EUNSUPPORTED;
     const int64_t cols = (int64_t)O * L;
     if ((cols + 255) / 256 > 0x7fffffffLL) return SFNO_EUNSUPPORTED;
-    hipLaunchKernelGGL(dhconv_colmax_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s, w, cmax, I, O, L, adjoint);
+    if ((I + DHF_CMAX_I - 1) / DHF_CMAX_I > 65535) return SFNO_EUNSUPPORTED;
+    hipLaunchKernelGGL(dhconv_colmax_clear_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s, cmax, cols);
+    hipLaunchKernelGGL(dhconv_colmax_kernel, dim3((unsigned)((cols + 255) / 256), (unsigned)((I + DHF_CMAX_I - 1) / DHF_CMAX_I)), dim3(256), 0, s, w, cmax, I,
+                       O, L, adjoint);
     const dim3 grid((unsigned)(nob * nc * ntc), (unsigned)((L + 7) / 8));
     if (ntc == 4)
         hipLaunchKernelGGL((dhconv_pack_f16_kernel<4>), grid, dim3(256), 0, s, w, cmax, reinterpret_cast<unsigned char*>(packed), cinv, I, O, L, nob, nc, adjoint);

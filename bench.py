@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SFNO spectral hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block|sfno8l|rollout|fft2_pair|pointwise_backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sht_pair|spectral_block|sfno8l|rollout|fft2_pair|pointwise_backward|train_step]
 
 Default workload (the configuration the headline metric is quoted on): forward + inverse
 real SHT at 721x1440 (equiangular, lmax = mmax = 721), batch 1, 73 channels, float32,
@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair", "pointwise_backward"])
+    ap.add_argument("--workload", default="sht_pair", choices=["sht_pair", "spectral_block", "sfno8l", "rollout", "fft2_pair", "pointwise_backward", "train_step"])
     ap.add_argument("--no-sfno", action="store_true", help="skip the SFNO-8L forward timing appended to the default run")
     ap.add_argument("--compute", default="fp32", choices=["fp32", "fp32_bf16x3", "bf16", "fp32_mfma"],
                     help="arithmetic of the Legendre and dhconv contractions: fp32 (reference precision: operands scaled and cut into two fp16 parts, "
@@ -790,6 +790,54 @@ def bench_pointwise_backward(args):
             "shapes": out}
 
 
+def bench_train_step(args):
+    """One training step of the SFNO-8L network (configs[3] shapes, batch 1) under bf16 autocast: forward, mean-square loss,
+    backward, SGD update (so that every packed weight copy is rebuilt each step, as in training).  The transforms, dhconv and
+    the 1x1 convolutions run on the HIP kernels in both directions; GELU and the instance norms are PyTorch's.  The same
+    step with the convolutions left to PyTorch's library kernels is timed beside it."""
+    import torch
+    from makani_amd import pointwise as pw
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    net = build_sfno8l(dev, args.compute).train()
+    opt = torch.optim.SGD(net.parameters(), lr=1e-6)
+    x = torch.randn(1, 73, 721, 1440, generator=torch.Generator().manual_seed(5)).to(dev)
+    tgt = torch.randn(1, 73, 721, 1440, generator=torch.Generator().manual_seed(6)).to(dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = net(x)
+        loss = ((y.float() - tgt) ** 2).mean()
+        loss.backward()
+        opt.step()
+        return loss
+
+    def timed():
+        for _ in range(max(args.warmup, 2)):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3, float(loss.detach())
+
+    ms, loss = timed()
+    peak = torch.cuda.max_memory_allocated() / 1e9
+    saved = pw.trainable_active
+    pw.trainable_active = lambda t: False
+    try:
+        ms_lib, _ = timed()
+    finally:
+        pw.trainable_active = saved
+    return {"metric": "SFNO-L8 training step ms/sample", "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 2),
+            "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 pointwise / f32 spectral", "data": "synthetic",
+            "config": {"workload": "SFNO-linear 8 layers, embed 384, 721x1440 -> 240x480, 73 channels, batch 1: forward + backward + SGD update, bf16 autocast"},
+            "ms_per_step_with_library_convolutions": ms_lib, "loss_finite": loss == loss and abs(loss) != float("inf"), "peak_memory_GB": peak}
+
+
 def legendre_fp32_mfma_figure(iters=10):
     """The Legendre stage of configs[1] on the fp32 matrix instruction (compute="fp32_mfma"): time per direction and algorithmic
     (triangular) flops over it against the fp32 MFMA peak."""
@@ -876,6 +924,8 @@ def main():
         res = bench_sfno8l(args)
     elif args.workload == "pointwise_backward":
         res = bench_pointwise_backward(args)
+    elif args.workload == "train_step":
+        res = bench_train_step(args)
     else:
         res = bench_rollout(args)
     print(json.dumps(res), flush=True)

@@ -27,3 +27,29 @@ def test_state_dict_keys_and_wiring(lib_built):
     w = net.state_dict()["blocks.1.filter.filter.weight"]
     assert tuple(w.shape) == (8, 8, 240) and w.dtype == torch.complex64
     assert tuple(net.state_dict()["blocks.0.mlp.fwd.0.weight"].shape) == (16, 8, 1, 1)
+
+
+def test_pointwise_convolutions_are_conv2d_modules_on_the_cpu(lib_built):
+    """The network's 1x1 convolutions are PointwiseConv2d modules: nn.Conv2d in everything a checkpoint or a CPU run sees
+    (class hierarchy, parameter names and shapes, values), the HIP route being taken only for bf16 HIP tensors with a gradient."""
+    import copy
+
+    from makani_amd import pointwise as pw
+    from makani_amd.sfnonet import SphericalFourierNeuralOperatorNet
+
+    torch.manual_seed(0)
+    net = SphericalFourierNeuralOperatorNet(inp_shape=(16, 32), out_shape=(16, 32), scale_factor=2, inp_chans=3, out_chans=2, embed_dim=8,
+                                            num_layers=2)
+    convs = [m for m in net.modules() if isinstance(m, torch.nn.Conv2d)]
+    assert convs and all(isinstance(m, pw.PointwiseConv2d) and m.kernel_size == (1, 1) for m in convs)
+    conv = convs[0]
+    ref = torch.nn.Conv2d(conv.in_channels, conv.out_channels, 1, bias=conv.bias is not None)
+    ref.load_state_dict(conv.state_dict())                      # same keys and shapes
+    x = torch.randn(2, conv.in_channels, 4, 8, requires_grad=True)
+    assert not pw.trainable_active(x)                           # CPU tensor: the module path
+    y = conv(x)
+    assert torch.equal(y, ref(x)) and not type(y.grad_fn).__name__.startswith("_Conv1x1")
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        assert not pw.trainable_active(x)
+    twin = copy.deepcopy(conv)
+    assert isinstance(twin, pw.PointwiseConv2d) and torch.equal(twin.weight, conv.weight)

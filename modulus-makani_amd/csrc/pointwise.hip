@@ -35,6 +35,14 @@ constexpr int PW_KALIGN = 128;    // K is padded to whole unrolled loop bodies (
 
 __device__ __forceinline__ float bf16_to_f(unsigned short h) { return __uint_as_float((unsigned int)h << 16); }
 __device__ __forceinline__ unsigned short f_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
+// two floats rounded to nearest-even bf16 in one word, lo in the low half (the hardware conversion takes a pair: one
+// instruction where two single conversions need a shift and an or as well)
+__device__ __forceinline__ unsigned int bf16_pair(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 f = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, bf16x2));
+}
 
 // p[i] for a wavefront-uniform i, of an array the kernel never writes: read through the scalar unit, whose loads do not
 // count against the vector memory counter
@@ -43,20 +51,21 @@ __device__ __forceinline__ float uniform_load(const float* p, int64_t i) {
 }
 
 // exact (erf) GELU for bf16 outputs.  gelu(x) = max(x, 0) - |x| erfc(|x| / sqrt 2) / 2 for both signs (no cancellation in
-// the negative tail), and erfc is evaluated as 2^Q(|x|): log2 erfc(t / sqrt 2) is smooth, a degree-7 polynomial in t follows it
-// to 7e-5 on [0, 8.5] (relative error of erfc 5e-5, a fortieth of the half ulp of the bf16 result); beyond 8.5 the term is
-// below 1e-16 and t is clamped.  Twelve full-rate instructions and one exp2, where a rational form needs a reciprocal as well.
+// the negative tail), and erfc is evaluated as 2^Q(|x|): log2 erfc(t / sqrt 2) is smooth, a degree-6 polynomial in t follows it
+// to 1.1e-4 on [0, 6.5] (relative error of erfc 7e-5, a thirtieth of the half ulp of the bf16 result).  Beyond 6.5 t is
+// clamped: the term is then below 3e-10 |x| / 6.5 in magnitude, where the formula x (1 + erf(x / sqrt 2)) / 2 in fp32
+// arithmetic has long returned -0.  Ten full-rate instructions and one exp2, where a rational form needs a reciprocal as well.
 __device__ __forceinline__ float gelu(float x) {
     // (the median of three stands for min and max: one instruction each, where fminf / fmaxf first canonicalise their operand)
-    const float t = __builtin_amdgcn_fmed3f(fabsf(x), 0.f, 8.5f);
-    float q = fmaf(t, -1.112324808e-06f, 4.422128154e-05f);
-    q = fmaf(t, q, -7.661478214e-04f);
-    q = fmaf(t, q, 7.736902644e-03f);
-    q = fmaf(t, q, -5.210667575e-02f);
-    q = fmaf(t, q, -4.605784664e-01f);
-    q = fmaf(t, q, -1.150352355e+00f);
-    q = fmaf(t, q, -5.705795628e-05f);
-    return fmaf(-0.5f * fabsf(x), __builtin_amdgcn_exp2f(q), __builtin_amdgcn_fmed3f(x, 0.f, __builtin_inff()));
+    const float t = __builtin_amdgcn_fmed3f(fabsf(x), 0.f, 6.5f);
+    float q = fmaf(t, 2.008575651e-05f, -5.615057212e-04f);
+    q = fmaf(t, q, 6.880626770e-03f);
+    q = fmaf(t, q, -5.027262948e-02f);
+    q = fmaf(t, q, -4.624537704e-01f);
+    q = fmaf(t, q, -1.149621597e+00f);
+    // (the factor 1/2 rides in the exponent: the constant term is the fitted -1.062872110e-04 minus one)
+    q = fmaf(t, q, -1.000106287211f);
+    return fmaf(-fabsf(x), __builtin_amdgcn_exp2f(q), __builtin_amdgcn_fmed3f(x, 0.f, __builtin_inff()));
 }
 
 // WM = wavefronts along the output rows: 4 (x 2 along pixels: 384 rows x 128 pixels per workgroup) or
@@ -245,7 +254,7 @@ __global__ __launch_bounds__(NT == 2 ? 512 : 256) void pw_gemm_kernel(PointwiseA
             }
             rw_t out;
 #pragma unroll
-            for (int pp = 0; pp < NT / 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
+            for (int pp = 0; pp < NT / 2; ++pp) out[pp] = bf16_pair(y[2 * pp], y[2 * pp + 1]);
             *reinterpret_cast<rw_t*>(Y + (int64_t)o * a.P + px) = out;
         }
     }
@@ -497,7 +506,7 @@ __global__ __launch_bounds__(512) void pw_gemm_dma_kernel(PointwiseArgs a) {
                     }
                     u32x2 out;
 #pragma unroll
-                    for (int pp = 0; pp < 2; ++pp) out[pp] = (unsigned int)f_to_bf16(y[2 * pp]) | ((unsigned int)f_to_bf16(y[2 * pp + 1]) << 16);
+                    for (int pp = 0; pp < 2; ++pp) out[pp] = bf16_pair(y[2 * pp], y[2 * pp + 1]);
                     *reinterpret_cast<u32x2*>(Y + (int64_t)row_of(mt, v) * a.P) = out;
                 }
             }
@@ -701,7 +710,7 @@ __global__ __launch_bounds__(256) void scale_shift_act_kernel(const unsigned sho
             lo = gelu(lo);
             hi = gelu(hi);
         }
-        o[i] = (unsigned int)f_to_bf16(lo) | ((unsigned int)f_to_bf16(hi) << 16);
+        o[i] = bf16_pair(lo, hi);
     }
     *reinterpret_cast<u32x4*>(y + i0) = o;
 }

@@ -158,3 +158,35 @@ def test_stream_leaves_out_only_negligible_polar_chunks(lib_built, nlat, lmax, m
     if nlat >= 241:
         assert kept < 0.95 * dense
     print(f"{grid} {nlat} lmax {lmax} mmax {mmax} {'analysis' if analysis else 'synthesis'}: {kept} of {dense} blocks kept")
+
+
+def test_pointwise_weight_grad_workspace_and_argument_checks(lib_built):
+    """Host side of sfno_pointwise_weight_grad: the workspace query (a whole number of [O][K + bias] partial matrices, one
+    per share of the pixel range: 8 to 256 shares, fewer for short inputs) and the argument checks that come before any launch."""
+    import ctypes
+
+    from makani_amd._lib import lib
+
+    q = lib.sfno_pointwise_weight_grad_workspace_bytes
+    for B, K, O, P, bias in [(1, 384, 768, 240 * 480, 1), (1, 768, 384, 240 * 480, 0), (2, 73, 384, 720, 1), (1, 1, 1, 8, 1), (4, 384, 73, 721 * 1440, 0),
+                             (1, 4096, 4096, 64, 1)]:
+        n = q(B, K, O, P, bias)
+        per = 4 * O * (K + bias)
+        assert n > 0 and n % per == 0, (B, K, O, P, bias, n)
+        shares = n // per
+        chunks = B * ((P + 31) // 32)
+        assert 1 <= shares <= 256 and shares <= max(1, (chunks + 7) // 8)
+        if chunks >= 8 * 256:
+            assert shares >= 8
+    # pixel counts the kernels do not take, and non-positive sizes: no workspace
+    for args in [(1, 8, 8, 12, 0), (1, 8, 8, 4, 0), (0, 8, 8, 64, 0), (1, 0, 8, 64, 0), (1, 8, 0, 64, 0)]:
+        assert q(*args) == 0
+    # null pointers, bad pixel counts and misaligned operands are refused before anything is launched
+    f = lib.sfno_pointwise_weight_grad
+    buf = ctypes.create_string_buffer(4096 + 64)
+    base = (ctypes.addressof(buf) + 63) & ~63
+    ok = ctypes.c_void_p(base)
+    assert f(None, ok, ok, None, 1, 8, 8, 64, ok, 4096, None) != 0
+    assert f(ok, ok, ok, None, 1, 8, 8, 12, ok, 4096, None) != 0
+    assert f(ctypes.c_void_p(base + 2), ok, ok, None, 1, 8, 8, 64, ok, 4096, None) != 0
+    assert f(ok, ok, ok, None, 1, 8, 8, 64, ctypes.c_void_p(base + 4), 4096, None) != 0

@@ -51,6 +51,7 @@ def parse():
     ap.add_argument("--batch", type=int, default=1, help="--workload spectral_block: samples per step (configs[2] is batch 1)")
     ap.add_argument("--backward", action="store_true", help="--workload spectral_block: time forward + backward (input and weight gradients)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-library-leg", action="store_true", help="--workload train_step: skip the same step with PyTorch's library convolutions")
     ap.add_argument("--yardstick", action="store_true",
                     help="also run one plain 256 MiB elementwise copy (mul by 1): the known-size reference for FETCH_SIZE/WRITE_SIZE runs")
     ap.add_argument("--cpu-sample-channels", type=int, default=4)
@@ -826,12 +827,14 @@ def bench_train_step(args):
 
     ms, loss = timed()
     peak = torch.cuda.max_memory_allocated() / 1e9
-    saved = pw.trainable_active
-    pw.trainable_active = lambda t: False
-    try:
-        ms_lib, _ = timed()
-    finally:
-        pw.trainable_active = saved
+    ms_lib = None
+    if not args.no_library_leg:
+        saved = pw.trainable_active
+        pw.trainable_active = lambda t: False
+        try:
+            ms_lib, _ = timed()
+        finally:
+            pw.trainable_active = saved
     return {"metric": "SFNO-L8 training step ms/sample", "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 2),
             "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 pointwise / f32 spectral", "data": "synthetic",
             "config": {"workload": "SFNO-linear 8 layers, embed 384, 721x1440 -> 240x480, 73 channels, batch 1: forward + backward + SGD update, bf16 autocast"},
